@@ -1,0 +1,444 @@
+"""Python face of libcutespmm.so (ctypes).  Class and field names follow the reference's
+host API: ``MTX_READER`` (IO.cu:2-88), ``HRPB`` (data.cu:54-340), ``SPMM_TC``
+(spmm.cu:258-840), ``check_gemm_correctness_coo`` (inc.h:84-109) and
+``GPU_CSR_cuSPARSE_NEW`` (spmm.cu:860-960, here a hand-written HIP CSR kernel).
+
+The shared library is the product; this module only marshals numpy arrays and device
+pointers into its C ABI.  There is no CPU fallback: device entry points raise
+``CuteError`` when the library or a gfx950 device is missing.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcutespmm.so")
+
+# every symbol declared in include/cutespmm.h
+ABI_SYMBOLS = [
+    "cute_status_string", "cute_last_hip_error", "cute_free",
+    "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
+    "cute_hrpb_build", "cute_hrpb_host_release",
+    "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
+    "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
+    "cute_gen_matrix", "cute_gen_dense",
+    "cute_hrpb_upload", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
+    "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run",
+    "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
+    "cute_device_info",
+]
+
+u32p = C.POINTER(C.c_uint32)
+u64p = C.POINTER(C.c_uint64)
+f32p = C.POINTER(C.c_float)
+
+
+class CuteError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = "%s: %s (%d)" % (where, _status_string(status), status)
+        if status == -7 or status == -8:
+            msg += " -- " + _last_hip_error()
+        super().__init__(msg)
+
+
+class cute_csr(C.Structure):
+    _fields_ = [("M", C.c_uint32), ("K", C.c_uint32), ("nnz", C.c_uint32),
+                ("rowPtr", u32p), ("cols", u32p), ("vals", f32p)]
+
+
+class cute_hrpb_host(C.Structure):
+    _fields_ = [("M", C.c_uint32), ("K", C.c_uint32), ("numRowPanels", C.c_uint32), ("numBlocks", C.c_uint32),
+                ("numWords", C.c_uint64), ("blockedRowPtr", u32p), ("activeCols", u32p), ("sizePtr", u64p),
+                ("blocksData", u32p), ("rowPtr", u32p), ("cols", u32p), ("vals", f32p),
+                ("nnz", C.c_uint32), ("numBricks", C.c_uint32)]
+
+
+class cute_hrpb_tiled(C.Structure):
+    _fields_ = [("M", C.c_uint32), ("K", C.c_uint32), ("numRowPanels", C.c_uint32), ("numBlocks", C.c_uint32),
+                ("numVals", C.c_uint64), ("blockedRowPtr", u32p), ("hdr", u32p), ("vals", f32p)]
+
+
+class cute_tunables(C.Structure):
+    _fields_ = [("path", C.c_int32), ("precision", C.c_int32), ("min_reuse", C.c_float), ("slots", C.c_uint32),
+                ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("reserved", C.c_uint32 * 2)]
+
+
+class cute_plan_info(C.Structure):
+    _fields_ = [("N", C.c_uint32), ("slabWidth", C.c_uint32), ("numSlabs", C.c_uint32), ("numChunks", C.c_uint32),
+                ("numAtomicChunks", C.c_uint32), ("numBrickPanels", C.c_uint32), ("numRowPanelsSparse", C.c_uint32),
+                ("numEmptyPanels", C.c_uint32), ("slots", C.c_uint32), ("precision", C.c_uint32),
+                ("path", C.c_uint32), ("reserved", C.c_uint32 * 5)]
+
+
+PATH_AUTO, PATH_BRICK, PATH_ROWS = 0, 1, 2
+PREC_FP32, PREC_BF16X3 = 0, 1
+
+_lib = None
+
+
+def load_library():
+    """Loads libcutespmm.so; raises if it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise CuteError(-8, "libcutespmm.so is not built (run python -m cutespmm_ae_amd.build); no fallback path")
+    lib = C.CDLL(LIB_PATH)
+    lib.cute_status_string.restype = C.c_char_p
+    lib.cute_status_string.argtypes = [C.c_int]
+    lib.cute_last_hip_error.restype = C.c_char_p
+    lib.cute_free.argtypes = [C.c_void_p]
+    lib.cute_mtx_read.argtypes = [C.c_char_p, C.c_int, C.POINTER(cute_csr)]
+    lib.cute_csr_release.argtypes = [C.POINTER(cute_csr)]
+    lib.cute_csr_sort_rows.argtypes = [C.POINTER(cute_csr)]
+    lib.cute_hrpb_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_hrpb_host)]
+    lib.cute_hrpb_host_release.argtypes = [C.POINTER(cute_hrpb_host)]
+    lib.cute_hrpb_retile.argtypes = [C.POINTER(cute_hrpb_host), C.POINTER(cute_hrpb_tiled)]
+    lib.cute_hrpb_untile.argtypes = [C.POINTER(cute_hrpb_tiled), C.POINTER(cute_hrpb_host)]
+    lib.cute_hrpb_tiled_release.argtypes = [C.POINTER(cute_hrpb_tiled)]
+    lib.cute_partition.restype = C.c_int64
+    lib.cute_partition.argtypes = [C.c_uint32, u32p, C.c_uint32, C.c_uint32, u32p, C.c_uint64]
+    lib.cute_check_gemm_correctness.restype = C.c_float
+    lib.cute_check_gemm_correctness.argtypes = [f32p, f32p, C.c_uint32, C.c_uint32]
+    lib.cute_backward_error.restype = C.c_float
+    lib.cute_backward_error.argtypes = [u32p, u32p, f32p, f32p, f32p, f32p, C.c_uint32, C.c_uint32]
+    lib.cute_gen_matrix.argtypes = [C.c_int, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(cute_csr)]
+    lib.cute_gen_dense.argtypes = [C.c_uint64, C.c_int, C.c_uint64, f32p]
+    lib.cute_hrpb_upload.argtypes = [C.POINTER(cute_hrpb_host), C.POINTER(C.c_void_p)]
+    lib.cute_hrpb_dev_free.argtypes = [C.c_void_p]
+    lib.cute_hrpb_dev_bytes.restype = C.c_uint64
+    lib.cute_hrpb_dev_bytes.argtypes = [C.c_void_p]
+    lib.cute_hrpb_dev_csr.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]
+    lib.cute_spmm_plan_create.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(cute_tunables), C.POINTER(C.c_void_p)]
+    lib.cute_spmm_plan_info.argtypes = [C.c_void_p, C.POINTER(cute_plan_info)]
+    lib.cute_spmm_plan_free.argtypes = [C.c_void_p]
+    lib.cute_spmm_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.cute_csr_spmm_dev.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_uint32, C.c_uint32, C.c_void_p]
+    lib.cute_gpu_csr_spmm.restype = C.c_float
+    lib.cute_gpu_csr_spmm.argtypes = [u32p, u32p, f32p, C.c_uint32, f32p, f32p, C.c_uint32, C.c_uint32, C.c_uint32,
+                                      C.c_int, C.c_int]
+    lib.cute_spmm_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, f32p]
+    lib.cute_csr_spmm_time.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p,
+                                       C.c_int, C.c_int, f32p]
+    lib.cute_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_size_t]
+    _lib = lib
+    return lib
+
+
+def _status_string(s):
+    try:
+        return load_library().cute_status_string(int(s)).decode()
+    except Exception:  # library missing: still produce a readable message
+        return "status"
+
+
+def _last_hip_error():
+    try:
+        return load_library().cute_last_hip_error().decode()
+    except Exception:
+        return ""
+
+
+def _check(rc, where):
+    if rc != 0:
+        raise CuteError(rc, where)
+
+
+def _as(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _ptr(a, t):
+    return a.ctypes.data_as(t)
+
+
+def _view(ptr, n, dtype):
+    n = int(n)
+    if n == 0:
+        return np.zeros(0, dtype)
+    return np.ctypeslib.as_array(ptr, shape=(n,)).view(dtype)
+
+
+# --------------------------------------------------------------------------------------
+# loaders / generators
+# --------------------------------------------------------------------------------------
+class CSR:
+    """Owner of a ``cute_csr``; fields M, K, nnz, rowPtr, cols, vals (numpy views)."""
+
+    def __init__(self, raw):
+        self._raw = raw
+        self.M, self.K, self.nnz = raw.M, raw.K, raw.nnz
+        self.rowPtr = _view(raw.rowPtr, raw.M + 1, np.uint32)
+        self.cols = _view(raw.cols, raw.nnz, np.uint32)
+        self.vals = _view(raw.vals, raw.nnz, np.float32)
+
+    def sort_rows(self):
+        _check(load_library().cute_csr_sort_rows(C.byref(self._raw)), "cute_csr_sort_rows")
+        return self
+
+    def __del__(self):
+        try:
+            load_library().cute_csr_release(C.byref(self._raw))
+        except Exception:
+            pass
+
+
+class MTX_READER(CSR):
+    """``MTX_READER(path)``: MatrixMarket file -> CSR with the reference's quirks
+    (dims padded to 16, symmetric mirrored, all values 1.0f unless ``keep_values``)."""
+
+    def __init__(self, file_path, keep_values=False):
+        raw = cute_csr()
+        _check(load_library().cute_mtx_read(os.fsencode(file_path), int(bool(keep_values)), C.byref(raw)),
+               "cute_mtx_read(%s)" % file_path)
+        super().__init__(raw)
+
+
+# stock parameters of the five benchmark configurations
+CONFIGS = {
+    1: dict(kind=1, p0=4096, p1=16, p2=0, N=32, name="uniform_4096_16nnz_N32"),
+    2: dict(kind=2, p0=256, p1=0, p2=0, N=128, name="stencil9_256x256_N128"),
+    3: dict(kind=3, p0=8000, p1=200, p2=0, N=128, name="fem_8000x6x6_N128"),
+    4: dict(kind=4, p0=17, p1=10, p2=0, N=64, name="rmat_2p17_deg10_N64"),
+    5: dict(kind=5, p0=1048576, p1=32, p2=2048, N=256, name="banded_1M_32nnz_N256"),
+}
+SEED_BASE = 0xC07E5B00
+
+
+def gen_matrix(kind, seed, p0, p1=0, p2=0):
+    raw = cute_csr()
+    _check(load_library().cute_gen_matrix(int(kind), C.c_uint64(seed), int(p0), int(p1), int(p2), C.byref(raw)),
+           "cute_gen_matrix")
+    return CSR(raw)
+
+
+def gen_config(cfg, scale=1.0):
+    """Matrix of benchmark configuration ``cfg`` (1..5); ``scale`` < 1 shrinks the row count."""
+    c = CONFIGS[cfg]
+    p0 = c["p0"]
+    if scale != 1.0:
+        if c["kind"] == 2:
+            p0 = max(16, int(p0 * scale ** 0.5) // 16 * 16)
+        elif c["kind"] == 4:
+            p0 = max(8, int(round(p0 + np.log2(scale))))
+        elif c["kind"] == 3:
+            p0 = max(64, int(p0 * scale) // 8 * 8)
+        else:
+            p0 = max(256, int(p0 * scale) // 16 * 16)
+    return gen_matrix(c["kind"], SEED_BASE + cfg, p0, c["p1"], c["p2"])
+
+
+def gen_dense(seed, rows, cols, dist=2):
+    """dist 0: U(0,1), 1: U(-1,1), 2: N(0,1).  Element i depends only on (seed, i)."""
+    out = np.empty((rows, cols), np.float32)
+    _check(load_library().cute_gen_dense(C.c_uint64(seed), int(dist), C.c_uint64(rows * cols), _ptr(out, f32p)),
+           "cute_gen_dense")
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# format
+# --------------------------------------------------------------------------------------
+class HRPB:
+    """``HRPB(M, K, rowPtr, cols, vals)``: canonical arrays as public fields
+    (blockedRowPtr, activeCols, sizePtr, blocksData, numRowPanels) as in data.cu:56-72.
+    ``upload()`` creates the device twin (data.cu:327-334); ``freeDevice()`` drops it."""
+
+    def __init__(self, M, K, rowPtr, cols, vals):
+        self.rowPtr = _as(rowPtr, np.uint32)
+        self.cols = _as(cols, np.uint32)
+        self.vals = _as(vals, np.float32)
+        self._raw = cute_hrpb_host()
+        self._dev = C.c_void_p()
+        _check(load_library().cute_hrpb_build(int(M), int(K), _ptr(self.rowPtr, u32p), _ptr(self.cols, u32p),
+                                              _ptr(self.vals, f32p), C.byref(self._raw)), "cute_hrpb_build")
+        r = self._raw
+        self.M, self.K = r.M, r.K
+        self.numRowPanels, self.numBlocks, self.numWords = r.numRowPanels, r.numBlocks, r.numWords
+        self.num_bricks, self.numNNZ = r.numBricks, r.nnz
+        self.blockedRowPtr = _view(r.blockedRowPtr, r.numRowPanels + 1, np.uint32)
+        self.activeCols = _view(r.activeCols, r.numBlocks * 16, np.uint32)
+        self.sizePtr = _view(r.sizePtr, r.numBlocks + 1, np.uint64)
+        self.blocksData = _view(r.blocksData, r.numWords, np.uint32)
+
+    def as_dict(self):
+        return dict(M=self.M, K=self.K, numRowPanels=self.numRowPanels, numBlocks=self.numBlocks,
+                    numWords=self.numWords, blockedRowPtr=self.blockedRowPtr, activeCols=self.activeCols,
+                    sizePtr=self.sizePtr, blocksData=self.blocksData)
+
+    def retile(self):
+        """Host copy of the MFMA-tiled device layout: dict(hdr[nb,32], vals, blockedRowPtr)."""
+        t = cute_hrpb_tiled()
+        _check(load_library().cute_hrpb_retile(C.byref(self._raw), C.byref(t)), "cute_hrpb_retile")
+        out = dict(numBlocks=t.numBlocks, numVals=t.numVals,
+                   hdr=_view(t.hdr, t.numBlocks * 32, np.uint32).reshape(-1, 32).copy(),
+                   vals=_view(t.vals, t.numVals, np.float32).copy(),
+                   blockedRowPtr=_view(t.blockedRowPtr, t.numRowPanels + 1, np.uint32).copy())
+        load_library().cute_hrpb_tiled_release(C.byref(t))
+        return out
+
+    def retile_roundtrip(self):
+        """retile then untile; returns the canonical arrays rebuilt from the tiled form."""
+        lib = load_library()
+        t, back = cute_hrpb_tiled(), cute_hrpb_host()
+        _check(lib.cute_hrpb_retile(C.byref(self._raw), C.byref(t)), "cute_hrpb_retile")
+        rc = lib.cute_hrpb_untile(C.byref(t), C.byref(back))
+        lib.cute_hrpb_tiled_release(C.byref(t))
+        _check(rc, "cute_hrpb_untile")
+        out = dict(numBlocks=back.numBlocks, numWords=back.numWords, nnz=back.nnz, numBricks=back.numBricks,
+                   blockedRowPtr=_view(back.blockedRowPtr, back.numRowPanels + 1, np.uint32).copy(),
+                   activeCols=_view(back.activeCols, back.numBlocks * 16, np.uint32).copy(),
+                   sizePtr=_view(back.sizePtr, back.numBlocks + 1, np.uint64).copy(),
+                   blocksData=_view(back.blocksData, back.numWords, np.uint32).copy())
+        lib.cute_hrpb_host_release(C.byref(back))
+        return out
+
+    def upload(self):
+        if not self._dev:
+            _check(load_library().cute_hrpb_upload(C.byref(self._raw), C.byref(self._dev)), "cute_hrpb_upload")
+        return self._dev
+
+    def device_bytes(self):
+        return load_library().cute_hrpb_dev_bytes(self._dev) if self._dev else 0
+
+    def freeDevice(self):
+        if self._dev:
+            load_library().cute_hrpb_dev_free(self._dev)
+            self._dev = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.freeDevice()
+            load_library().cute_hrpb_host_release(C.byref(self._raw))
+        except Exception:
+            pass
+
+
+def partition(blockedRowPtr, nbN, slots):
+    """spmm.cu:776-812 arithmetic -> uint32 [n,4] {start, end, panel, atomic}."""
+    brp = _as(blockedRowPtr, np.uint32)
+    P = len(brp) - 1
+    lib = load_library()
+    n = lib.cute_partition(P, _ptr(brp, u32p), int(nbN), int(slots), None, 0)
+    if n < 0:
+        raise CuteError(int(n), "cute_partition")
+    out = np.zeros((max(n, 1), 4), np.uint32)
+    lib.cute_partition(P, _ptr(brp, u32p), int(nbN), int(slots), _ptr(out, u32p), n)
+    return out[:n]
+
+
+# --------------------------------------------------------------------------------------
+# plan + launch
+# --------------------------------------------------------------------------------------
+def _dev_ptr(t):
+    import torch
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+        raise TypeError("expected a contiguous float32 tensor on the GPU")
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream_ptr(stream):
+    import torch
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+class SPMM_TC:
+    """``SPMM_TC(hrpb, N)`` plans (spmm.cu:276-822); ``run(MatB, MatC)`` launches
+    (spmm.cu:823-839) on torch's current stream.  MatB [K,N], MatC [M,N] float32 GPU tensors."""
+
+    def __init__(self, hrpb, N, path=PATH_AUTO, precision=PREC_FP32, min_reuse=0.0, slots=0, max_chunk_blocks=0,
+                 brick_groups=0):
+        self.hrpb = hrpb
+        self.M, self.K, self.N = hrpb.M, hrpb.K, int(N)
+        self._plan = C.c_void_p()
+        t = cute_tunables(path=path, precision=precision, min_reuse=min_reuse, slots=slots,
+                          max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups)
+        _check(load_library().cute_spmm_plan_create(hrpb.upload(), self.N, C.byref(t), C.byref(self._plan)),
+               "cute_spmm_plan_create")
+        info = cute_plan_info()
+        _check(load_library().cute_spmm_plan_info(self._plan, C.byref(info)), "cute_spmm_plan_info")
+        self.info = {k: getattr(info, k) for k, _ in cute_plan_info._fields_ if k != "reserved"}
+        self.numRowPanelsSplit = info.numChunks
+
+    def _check_shapes(self, MatB, MatC):
+        if tuple(MatB.shape) != (self.K, self.N) or tuple(MatC.shape) != (self.M, self.N):
+            raise ValueError("MatB must be [%d,%d] and MatC [%d,%d]" % (self.K, self.N, self.M, self.N))
+
+    def run(self, MatB, MatC, stream=None):
+        self._check_shapes(MatB, MatC)
+        _check(load_library().cute_spmm_run(self._plan, _dev_ptr(MatB), _dev_ptr(MatC), _stream_ptr(stream)),
+               "cute_spmm_run")
+        return MatC
+
+    def time(self, MatB, MatC, warmup=3, iters=20, stream=None):
+        """Per-launch milliseconds (HIP events on the launch stream)."""
+        self._check_shapes(MatB, MatC)
+        ms = np.zeros(iters, np.float32)
+        _check(load_library().cute_spmm_time(self._plan, _dev_ptr(MatB), _dev_ptr(MatC), _stream_ptr(stream),
+                                             int(warmup), int(iters), _ptr(ms, f32p)), "cute_spmm_time")
+        return ms
+
+    def __del__(self):
+        try:
+            if self._plan:
+                load_library().cute_spmm_plan_free(self._plan)
+        except Exception:
+            pass
+
+
+def csr_spmm_time(alg, hrpb, MatB, MatC, warmup=3, iters=20, stream=None):
+    ms = np.zeros(iters, np.float32)
+    _check(load_library().cute_csr_spmm_time(int(alg), hrpb.upload(), _dev_ptr(MatB), _dev_ptr(MatC),
+                                             int(MatB.shape[1]), _stream_ptr(stream), int(warmup), int(iters),
+                                             _ptr(ms, f32p)), "cute_csr_spmm_time")
+    return ms
+
+
+def csr_spmm_dev(alg, hrpb, MatB, MatC, stream=None):
+    lib = load_library()
+    rp, cl, vl = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _check(lib.cute_hrpb_dev_csr(hrpb.upload(), C.byref(rp), C.byref(cl), C.byref(vl)), "cute_hrpb_dev_csr")
+    _check(lib.cute_csr_spmm_dev(int(alg), rp, cl, vl, _dev_ptr(MatB), _dev_ptr(MatC), hrpb.M, int(MatB.shape[1]),
+                                 _stream_ptr(stream)), "cute_csr_spmm_dev")
+    return MatC
+
+
+def GPU_CSR_cuSPARSE_NEW(rowPtr, cols, vals, nnz, hB, hC, m, k, n, iters, alg=2):
+    """Host arrays in, host C out, returns ms per launch (signature of spmm.cu:860-861)."""
+    rowPtr, cols, vals = _as(rowPtr, np.uint32), _as(cols, np.uint32), _as(vals, np.float32)
+    hB = _as(hB, np.float32)
+    assert hC.dtype == np.float32 and hC.flags.c_contiguous
+    ms = load_library().cute_gpu_csr_spmm(_ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p), int(nnz),
+                                          _ptr(hB, f32p), _ptr(hC, f32p), int(m), int(k), int(n), int(iters), int(alg))
+    if ms < 0:
+        raise CuteError(int(ms), "cute_gpu_csr_spmm")
+    return ms
+
+
+# --------------------------------------------------------------------------------------
+# metrics
+# --------------------------------------------------------------------------------------
+def check_gemm_correctness_coo(C_ref, C_test, M=None, N=None):
+    a, b = _as(C_ref, np.float32), _as(C_test, np.float32)
+    M = a.shape[0] if M is None else M
+    N = a.shape[1] if N is None else N
+    return float(load_library().cute_check_gemm_correctness(_ptr(a, f32p), _ptr(b, f32p), int(M), int(N)))
+
+
+def backward_error(rowPtr, cols, vals, B, C_ref, C_test):
+    rowPtr, cols, vals = _as(rowPtr, np.uint32), _as(cols, np.uint32), _as(vals, np.float32)
+    B, a, b = _as(B, np.float32), _as(C_ref, np.float32), _as(C_test, np.float32)
+    return float(load_library().cute_backward_error(_ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p),
+                                                    _ptr(B, f32p), _ptr(a, f32p), _ptr(b, f32p),
+                                                    len(rowPtr) - 1, B.shape[1]))
+
+
+def device_info():
+    cus, ws = C.c_int(), C.c_int()
+    name = C.create_string_buffer(64)
+    _check(load_library().cute_device_info(C.byref(cus), C.byref(ws), name, 64), "cute_device_info")
+    return dict(num_cus=cus.value, wave_size=ws.value, arch=name.value.decode())

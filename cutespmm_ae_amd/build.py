@@ -1,0 +1,62 @@
+"""Builds libcutespmm.so (gfx950 only) and the C++ driver with hipcc, in-tree."""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+ROOT = os.path.dirname(HERE)
+LIB = os.path.join(HERE, "libcutespmm.so")
+DRIVER = os.path.join(HERE, "run_cute")
+
+HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+# -packed-fp32-ops is switched off for device code: the compiler then never forms
+# v_pk_{add,mul,fma}_f32 from scalar float code.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-munsafe-fp-atomics"]
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+          "-pthread"]
+
+LIB_SOURCES = ["host_format.cpp", "gen.cpp", "device.hip"]
+
+
+def _run(cmd):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_library():
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    for s in LIB_SOURCES:
+        path = os.path.join(CSRC, s)
+        obj = os.path.join(objdir, s + ".o")
+        if s.endswith(".cpp"):               # host-only translation units
+            _run([HIPCC, "-x", "c++", path, "-c", "-o", obj] + COMMON)
+        else:
+            _run([HIPCC, "-x", "hip", path, "-c", "-o", obj] + COMMON + DEVICE_FLAGS)
+        objs.append(obj)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-pthread", "-o", LIB] + objs)
+    return LIB
+
+
+def build_driver():
+    src = os.path.join(CSRC, "run_cute.cpp")
+    if not os.path.exists(src):
+        return None
+    _run([HIPCC, "-x", "c++", src] + COMMON + ["-I", os.path.join(ROOT, "include"), "-o", DRIVER,
+                                                "-L", HERE, "-lcutespmm", "-Wl,-rpath,$ORIGIN"])
+    return DRIVER
+
+
+def build_all():
+    build_library()
+    build_driver()
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

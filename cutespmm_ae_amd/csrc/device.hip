@@ -1,0 +1,484 @@
+// Device side of libcutespmm: upload, plan, launch, plain CSR kernels, timing helpers.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <string>
+
+#include "common.hpp"
+#include "kernels.hip.hpp"
+
+using namespace cute;
+
+namespace {
+
+thread_local std::string g_hip_error;
+
+inline int hip_fail(hipError_t e, const char *what, int line)
+{
+    g_hip_error = std::string(hipGetErrorString(e)) + " (" + what + ", device.hip:" + std::to_string(line) + ")";
+    return CUTE_ERR_HIP;
+}
+#define HIP_TRY(expr)                                                    \
+    do {                                                                 \
+        hipError_t e_ = (expr);                                          \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr, __LINE__);      \
+    } while (0)
+
+struct DeviceContext {
+    int status = CUTE_ERR_NO_DEVICE;
+    int device = 0;
+    int num_cus = 0;
+    int wave_size = 0;
+    std::string arch;
+};
+
+// The library is written for gfx950 only; any other device is refused, loudly.
+const DeviceContext &context()
+{
+    static DeviceContext ctx = [] {
+        DeviceContext c;
+        int n = 0;
+        if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+            g_hip_error = "no HIP device visible";
+            return c;
+        }
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return c;
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return c;
+        c.device = dev;
+        c.num_cus = prop.multiProcessorCount;
+        c.wave_size = prop.warpSize;
+        c.arch = prop.gcnArchName;
+        if (c.arch.rfind("gfx950", 0) != 0) {
+            g_hip_error = "device is " + c.arch + ", this library is built for gfx950 only";
+            return c;
+        }
+        c.status = CUTE_OK;
+        return c;
+    }();
+    return ctx;
+}
+
+template <class T>
+int upload(T **dst, const T *src, uint64_t count)
+{
+    *dst = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), std::max<uint64_t>(count, 1) * sizeof(T)));
+    if (count) HIP_TRY(hipMemcpy(*dst, src, count * sizeof(T), hipMemcpyHostToDevice));
+    return CUTE_OK;
+}
+
+}  // namespace
+
+struct cute_hrpb_dev {
+    uint32_t M = 0, K = 0, nnz = 0, P = 0, nb = 0;
+    uint64_t numVals = 0, bytes = 0;
+    uint32_t *dHdr = nullptr;
+    float *dVals = nullptr;
+    uint32_t *dRowPtr = nullptr, *dCols = nullptr;
+    float *dCsrVals = nullptr;
+    std::vector<uint32_t> brp;          // host copy of blockedRowPtr
+    std::vector<uint32_t> panelNnz;     // nonzeros per row panel
+    std::vector<uint32_t> panelCols;    // active columns per row panel
+};
+
+struct cute_spmm_plan {
+    const cute_hrpb_dev *d = nullptr;
+    cute_plan_info info{};
+    int vec = 4, ng = 1;                // brick kernel shape
+    int rows_vec = 4, rows_logl = 6;    // row kernel shape
+    uint32_t rows_slabs = 1;
+    uint4 *dChunks = nullptr;
+    uint32_t *dAtomicPanels = nullptr;
+    uint32_t numAtomicPanels = 0;
+    uint32_t *dRowList = nullptr;
+    uint32_t numRows = 0;
+};
+
+extern "C" {
+
+const char *cute_last_hip_error(void) { return g_hip_error.c_str(); }
+
+int cute_device_info(int *num_cus, int *wave_size, char *arch_name, size_t arch_cap)
+{
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    if (num_cus) *num_cus = c.num_cus;
+    if (wave_size) *wave_size = c.wave_size;
+    if (arch_name && arch_cap) std::snprintf(arch_name, arch_cap, "%s", c.arch.c_str());
+    return CUTE_OK;
+}
+
+void cute_hrpb_dev_free(cute_hrpb_dev *d)
+{
+    if (!d) return;
+    (void)hipFree(d->dHdr);
+    (void)hipFree(d->dVals);
+    (void)hipFree(d->dRowPtr);
+    (void)hipFree(d->dCols);
+    (void)hipFree(d->dCsrVals);
+    delete d;
+}
+
+uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d) { return d ? d->bytes : 0; }
+
+int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
+{
+    if (!h || !out || !h->rowPtr) return CUTE_ERR_ARG;
+    *out = nullptr;
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    cute_hrpb_tiled t;
+    int rc = cute_hrpb_retile(h, &t);
+    if (rc != CUTE_OK) return rc;
+    cute_hrpb_dev *d = new cute_hrpb_dev;
+    d->M = h->M;
+    d->K = h->K;
+    d->nnz = h->nnz;
+    d->P = h->numRowPanels;
+    d->nb = h->numBlocks;
+    d->numVals = t.numVals;
+    d->brp.assign(h->blockedRowPtr, h->blockedRowPtr + h->numRowPanels + 1);
+    d->panelNnz.resize(d->P);
+    d->panelCols.resize(d->P);
+    for (uint32_t p = 0; p < d->P; ++p) {
+        d->panelNnz[p] = h->rowPtr[(p + 1) * CUTE_TM] - h->rowPtr[p * CUTE_TM];
+        const uint32_t nblk = d->brp[p + 1] - d->brp[p];
+        uint32_t live = 0;
+        if (nblk) {
+            const uint32_t *hd = t.hdr + uint64_t(d->brp[p + 1] - 1) * CUTE_TILED_HDR_WORDS;
+            for (uint32_t j = 0; j < 4; ++j) {
+                uint64_t bm;
+                std::memcpy(&bm, hd + 16 + 2 * j, 8);
+                for (uint32_t k = 0; k < 4; ++k) live += ((bm >> (16 * k)) & 0xFFFFull) ? 1u : 0u;
+            }
+            live += (nblk - 1) * CUTE_TK;
+        }
+        d->panelCols[p] = live;
+    }
+    rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
+    if (rc == CUTE_OK) rc = upload(&d->dVals, t.vals, t.numVals);
+    if (rc == CUTE_OK) rc = upload(&d->dRowPtr, h->rowPtr, uint64_t(h->M) + 1);
+    if (rc == CUTE_OK) rc = upload(&d->dCols, h->cols, h->nnz);
+    if (rc == CUTE_OK) rc = upload(&d->dCsrVals, h->vals, h->nnz);
+    d->bytes = uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + t.numVals * 4 + (uint64_t(h->M) + 1) * 4 +
+               uint64_t(h->nnz) * 8;
+    cute_hrpb_tiled_release(&t);
+    if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
+    *out = d;
+    return CUTE_OK;
+}
+
+int cute_hrpb_dev_csr(const cute_hrpb_dev *d, const uint32_t **dRowPtr, const uint32_t **dCols, const float **dVals)
+{
+    if (!d) return CUTE_ERR_ARG;
+    if (dRowPtr) *dRowPtr = d->dRowPtr;
+    if (dCols) *dCols = d->dCols;
+    if (dVals) *dVals = d->dCsrVals;
+    return CUTE_OK;
+}
+
+void cute_spmm_plan_free(cute_spmm_plan *p)
+{
+    if (!p) return;
+    (void)hipFree(p->dChunks);
+    (void)hipFree(p->dAtomicPanels);
+    (void)hipFree(p->dRowList);
+    delete p;
+}
+
+int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out)
+{
+    if (!p || !out) return CUTE_ERR_ARG;
+    *out = p->info;
+    return CUTE_OK;
+}
+
+// Replaces SPMM_TC's constructor chain (spmm.cu:276-822).  The per-N launch shapes of
+// spmm.cu:11-101 and the occupancy table of spmm.cu:290-690 describe NVIDIA parts; here
+// the shape follows from wave64 MFMA tiles (16 lanes x VEC columns per group) and the slot
+// count from the CU count of the device.
+int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn, cute_spmm_plan **out)
+{
+    if (!d || !out) return CUTE_ERR_ARG;
+    *out = nullptr;
+    if (N == 0) return CUTE_ERR_SHAPE;
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    cute_tunables t{};
+    if (tn) t = *tn;
+    if (t.path < CUTE_PATH_AUTO || t.path > CUTE_PATH_ROWS) return CUTE_ERR_ARG;
+    if (t.precision != CUTE_PREC_FP32) return CUTE_ERR_ARG;   // the bf16x3 kernel is not built yet
+    const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : 1.25f;
+
+    cute_spmm_plan *p = new cute_spmm_plan;
+    p->d = d;
+    // brick kernel shape
+    p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    p->ng = (p->vec == 4 && N >= 128) ? 2 : 1;
+    if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
+    const uint32_t slab = 16u * p->vec * p->ng;
+    const uint32_t num_slabs = (N + slab - 1) / slab;
+    // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
+    p->rows_vec = p->vec;
+    {
+        uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
+        while ((1u << logl) < need && logl < 6) ++logl;
+        p->rows_logl = int(logl);
+        const uint32_t w = (1u << logl) * p->rows_vec;
+        p->rows_slabs = (N + w - 1) / w;
+    }
+
+    // classify panels
+    std::vector<uint8_t> to_rows(d->P, 0);
+    uint32_t n_brick = 0, n_rows = 0, n_empty = 0;
+    for (uint32_t q = 0; q < d->P; ++q) {
+        const uint32_t nblk = d->brp[q + 1] - d->brp[q];
+        bool rows;
+        if (nblk == 0) { rows = true; n_empty++; }
+        else if (t.path == CUTE_PATH_BRICK) rows = false;
+        else if (t.path == CUTE_PATH_ROWS) rows = true;
+        else rows = float(d->panelNnz[q]) < min_reuse * float(d->panelCols[q]);
+        to_rows[q] = rows;
+        if (nblk) (rows ? n_rows : n_brick)++;
+    }
+
+    // chunk list for the brick kernel
+    const uint32_t slots = t.slots ? t.slots : uint32_t(c.num_cus) * 4u * 4u;   // 4 SIMDs x 4 wavefronts
+    std::vector<uint32_t> quads;
+    {
+        int64_t n = cute_partition(d->P, d->brp.data(), num_slabs, slots, nullptr, 0);
+        if (n < 0) { delete p; return int(n); }
+        quads.resize(uint64_t(n) * 4);
+        cute_partition(d->P, d->brp.data(), num_slabs, slots, quads.data(), uint64_t(n));
+    }
+    std::vector<uint4> chunks;
+    std::vector<uint32_t> atomic_panels;
+    uint32_t n_atomic = 0;
+    for (size_t i = 0; i + 3 < quads.size(); i += 4) {
+        const uint32_t s = quads[i], e = quads[i + 1], pan = quads[i + 2];
+        uint32_t atomic = quads[i + 3];
+        if (to_rows[pan]) continue;
+        const uint32_t len = e - s;
+        const uint32_t cap = t.max_chunk_blocks ? t.max_chunk_blocks : len;
+        if (len > cap) atomic = 1;                 // cut further than the partition asked for
+        const uint32_t step = std::min(cap, len);
+        if (atomic && (atomic_panels.empty() || atomic_panels.back() != pan)) atomic_panels.push_back(pan);
+        for (uint32_t cs = s; cs < e; cs += step) {
+            chunks.push_back(make_uint4(cs, std::min(e, cs + step), pan, atomic));
+            n_atomic += atomic;
+        }
+    }
+    // panels ascend through the chunk list, so each atomic panel is listed (and zeroed) once
+    std::vector<uint32_t> row_list;
+    for (uint32_t q = 0; q < d->P; ++q)
+        if (to_rows[q])
+            for (uint32_t r = 0; r < CUTE_TM; ++r) row_list.push_back(q * CUTE_TM + r);
+
+    int rc = upload(&p->dChunks, chunks.data(), chunks.size());
+    if (rc == CUTE_OK) rc = upload(&p->dAtomicPanels, atomic_panels.data(), atomic_panels.size());
+    if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
+    if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
+    p->numAtomicPanels = uint32_t(atomic_panels.size());
+    p->numRows = uint32_t(row_list.size());
+    p->info.N = N;
+    p->info.slabWidth = slab;
+    p->info.numSlabs = num_slabs;
+    p->info.numChunks = uint32_t(chunks.size());
+    p->info.numAtomicChunks = n_atomic;
+    p->info.numBrickPanels = n_brick;
+    p->info.numRowPanelsSparse = n_rows;
+    p->info.numEmptyPanels = n_empty;
+    p->info.slots = slots;
+    p->info.precision = uint32_t(t.precision);
+    p->info.path = uint32_t(t.path);
+    *out = p;
+    return CUTE_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+template <int VEC, int NG>
+void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+{
+    const uint64_t items = uint64_t(p->info.numChunks) * p->info.numSlabs;
+    const uint32_t groups = uint32_t((items + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup);
+    const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG>), dim3(per_xcd * cute_dev::kNumXcd),
+                       dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
+                       p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+}
+
+template <int VEC>
+void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
+                     const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
+{
+    const uint64_t lanes = (uint64_t(num_rows) * slabs) << logl;
+    const dim3 grid(uint32_t((lanes + 255) / 256)), block(256);
+#define CUTE_ROWS_CASE(LL)                                                                                        \
+    case LL:                                                                                                      \
+        hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, row_list, num_rows, slabs, rp, cl, vl, \
+                           dB, dC, N);                                                                            \
+        break;
+    switch (logl) {
+        CUTE_ROWS_CASE(0) CUTE_ROWS_CASE(1) CUTE_ROWS_CASE(2) CUTE_ROWS_CASE(3)
+        CUTE_ROWS_CASE(4) CUTE_ROWS_CASE(5) CUTE_ROWS_CASE(6)
+    }
+#undef CUTE_ROWS_CASE
+}
+
+void launch_rows(int vec, int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
+                 const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
+{
+    if (vec == 4) launch_rows_vec<4>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    else if (vec == 2) launch_rows_vec<2>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    else launch_rows_vec<1>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+}
+
+int check_launch(const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, what, __LINE__);
+    return CUTE_OK;
+}
+
+int csr_launch(int alg, const uint32_t *rp, const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t M,
+               uint32_t N, hipStream_t s)
+{
+    if (M == 0 || N == 0) return CUTE_ERR_SHAPE;
+    switch (alg) {
+        case 0:
+            hipLaunchKernelGGL(cute_dev::csr_thread_per_element, dim3((N + 63) / 64, (M + 3) / 4), dim3(64, 4), 0, s, rp,
+                               cl, vl, dB, dC, M, N);
+            break;
+        case 1:
+            hipLaunchKernelGGL(cute_dev::csr_wave_scalar, dim3(uint32_t((uint64_t(M) * 64 + 255) / 256)), dim3(256), 0,
+                               s, rp, cl, vl, dB, dC, M, N);
+            break;
+        case 2: {
+            const int vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+            uint32_t need = (N + vec - 1) / vec, logl = 0;
+            while ((1u << logl) < need && logl < 6) ++logl;
+            const uint32_t w = (1u << logl) * vec;
+            launch_rows(vec, int(logl), nullptr, M, (N + w - 1) / w, rp, cl, vl, dB, dC, N, s);
+            break;
+        }
+        default: return CUTE_ERR_ARG;
+    }
+    return check_launch("csr kernel launch");
+}
+
+}  // namespace
+
+namespace {
+template <class Launch>
+int time_launches(hipStream_t s, int warmup, int iters, float *ms_out, Launch launch)
+{
+    if (iters < 1 || !ms_out) return CUTE_ERR_ARG;
+    std::vector<hipEvent_t> ev(size_t(iters) * 2, nullptr);
+    for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+    int rc = CUTE_OK;
+    for (int i = 0; i < warmup && rc == CUTE_OK; ++i) rc = launch();
+    for (int i = 0; i < iters && rc == CUTE_OK; ++i) {
+        (void)hipEventRecord(ev[2 * i], s);
+        rc = launch();
+        (void)hipEventRecord(ev[2 * i + 1], s);
+    }
+    if (rc == CUTE_OK && hipStreamSynchronize(s) != hipSuccess) rc = CUTE_ERR_HIP;
+    for (int i = 0; i < iters && rc == CUTE_OK; ++i)
+        if (hipEventElapsedTime(&ms_out[i], ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = CUTE_ERR_HIP;
+    for (auto &e : ev) (void)hipEventDestroy(e);
+    return rc;
+}
+}  // namespace
+
+extern "C" {
+
+// Replaces SPMM_TC::run (spmm.cu:823-839): picks the kernel instantiation from N and
+// launches asynchronously on `stream`.
+int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
+{
+    if (!p || !dB || !dC) return CUTE_ERR_ARG;
+    if ((reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC)) & 15u) return CUTE_ERR_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t N = p->info.N;
+    if (p->numAtomicPanels) {
+        hipLaunchKernelGGL(cute_dev::zero_panels, dim3(p->numAtomicPanels), dim3(256), 0, s, p->dAtomicPanels,
+                           p->numAtomicPanels, dC, N);
+    }
+    if (p->info.numChunks) {
+        if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
+        else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);
+        else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, s);
+        else launch_brick<1, 1>(p, dB, dC, s);
+    }
+    if (p->numRows) {
+        launch_rows(p->rows_vec, p->rows_logl, p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
+                    p->d->dCsrVals, dB, dC, N, s);
+    }
+    return check_launch("spmm launch");
+}
+
+int cute_csr_spmm_dev(int alg, const uint32_t *dRowPtr, const uint32_t *dCols, const float *dVals, const float *dB,
+                      float *dC, uint32_t M, uint32_t N, void *stream)
+{
+    if (!dRowPtr || !dB || !dC) return CUTE_ERR_ARG;
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    return csr_launch(alg, dRowPtr, dCols, dVals, dB, dC, M, N, static_cast<hipStream_t>(stream));
+}
+
+// Shape of GPU_CSR_cuSPARSE_NEW (spmm.cu:860-960): host arrays in, host C out, one warm-up
+// launch then `iters` timed launches between two events; returns ms per launch.
+float cute_gpu_csr_spmm(const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t nnz, const float *hB,
+                        float *hC, uint32_t m, uint32_t k, uint32_t n, int iters, int alg)
+{
+    if (!rowPtr || !hB || !hC || iters < 1) return -float(-CUTE_ERR_ARG);
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return float(c.status);
+    uint32_t *dR = nullptr, *dCl = nullptr;
+    float *dV = nullptr, *dB = nullptr, *dC = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    float ms = 0.0f;
+    int rc = upload(&dR, rowPtr, uint64_t(m) + 1);
+    if (rc == CUTE_OK) rc = upload(&dCl, cols, nnz);
+    if (rc == CUTE_OK) rc = upload(&dV, vals, nnz);
+    if (rc == CUTE_OK) rc = upload(&dB, hB, uint64_t(k) * n);
+    if (rc == CUTE_OK && hipMalloc(reinterpret_cast<void **>(&dC), uint64_t(m) * n * sizeof(float)) != hipSuccess)
+        rc = CUTE_ERR_HIP;
+    if (rc == CUTE_OK) rc = csr_launch(alg, dR, dCl, dV, dB, dC, m, n, nullptr);
+    if (rc == CUTE_OK && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = CUTE_ERR_HIP;
+    if (rc == CUTE_OK) {
+        (void)hipEventRecord(e0, nullptr);
+        for (int i = 0; i < iters && rc == CUTE_OK; ++i) rc = csr_launch(alg, dR, dCl, dV, dB, dC, m, n, nullptr);
+        (void)hipEventRecord(e1, nullptr);
+        if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess) rc = CUTE_ERR_HIP;
+    }
+    if (rc == CUTE_OK && hipMemcpy(hC, dC, uint64_t(m) * n * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
+        rc = CUTE_ERR_HIP;
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(dR); (void)hipFree(dCl); (void)hipFree(dV); (void)hipFree(dB); (void)hipFree(dC);
+    return rc == CUTE_OK ? ms / float(iters) : float(rc);
+}
+
+int cute_spmm_time(cute_spmm_plan *p, const float *dB, float *dC, void *stream, int warmup, int iters, float *ms_out)
+{
+    if (!p) return CUTE_ERR_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return time_launches(s, warmup, iters, ms_out, [&] { return cute_spmm_run(p, dB, dC, stream); });
+}
+
+int cute_csr_spmm_time(int alg, const cute_hrpb_dev *d, const float *dB, float *dC, uint32_t N, void *stream, int warmup,
+                       int iters, float *ms_out)
+{
+    if (!d) return CUTE_ERR_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return time_launches(s, warmup, iters, ms_out,
+                         [&] { return csr_launch(alg, d->dRowPtr, d->dCols, d->dCsrVals, dB, dC, d->M, N, s); });
+}
+
+}  // extern "C"

@@ -1,0 +1,260 @@
+// gfx950 device kernels of libcutespmm.
+//
+//   hrpb_brick_f32   one wavefront per (row-panel chunk, N slab); every non-empty 16x4
+//                    brick is one v_mfma_f32_16x16x4_f32 A operand taken straight from the
+//                    lane-order bitmap; B rows are gathered in the MFMA B-operand layout
+//                    (16 lanes read one contiguous row segment) so no LDS transpose is needed.
+//   csr_rows         one lane group per CSR row, lanes span N, (col, val) pairs broadcast
+//                    by lane shuffles; used for sparse panels and as a plain CSR kernel.
+//   csr_thread_per_element / csr_wave_scalar   the simple CSR comparison kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cute_dev {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+template <int VEC> struct Vec;
+template <> struct Vec<1> { typedef float type; };
+template <> struct Vec<2> { typedef f32x2 type; };
+template <> struct Vec<4> { typedef f32x4 type; };
+
+template <int VEC> __device__ __forceinline__ float vec_get(const typename Vec<VEC>::type &v, int i) { return v[i]; }
+template <> __device__ __forceinline__ float vec_get<1>(const float &v, int) { return v; }
+template <int VEC> __device__ __forceinline__ void vec_set(typename Vec<VEC>::type &v, int i, float x) { v[i] = x; }
+template <> __device__ __forceinline__ void vec_set<1>(float &v, int, float x) { v = x; }
+
+constexpr int kWaveSize = 64;
+constexpr int kWavesPerGroup = 4;
+constexpr int kHdrWords = 32;
+constexpr int kNumXcd = 8;
+
+// Work-groups are handed to the 8 XCDs round-robin; this maps the hardware id to a
+// logical id such that each XCD walks one contiguous range of logical ids (neighbouring
+// row panels share B rows, which then stay in that XCD's L2).
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t groups_per_xcd)
+{
+    return (bid % kNumXcd) * groups_per_xcd + bid / kNumXcd;
+}
+
+struct BlockHeader {          // wave-uniform part of one 128-byte header line
+    uint64_t bitmap[4];
+    uint32_t voff[4];
+};
+
+template <int VEC, int NG>
+struct BlockOperands {
+    float a[4];                                   // A operand per brick (lane L <-> bitmap bit L)
+    typename Vec<VEC>::type b[4][NG];             // B operand vectors per brick and column group
+    uint64_t live;                                // bit j set: brick j is non-empty (wave-uniform)
+};
+
+__device__ __forceinline__ BlockHeader load_header(const uint32_t *__restrict__ hdr, uint32_t blk)
+{
+    const uint32_t *h = hdr + size_t(blk) * kHdrWords;
+    BlockHeader r;
+    const uint64_t *bm = reinterpret_cast<const uint64_t *>(h + 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.bitmap[j] = bm[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.voff[j] = h[24 + j];
+    return r;
+}
+
+template <int VEC, int NG>
+__device__ __forceinline__ void load_operands(BlockOperands<VEC, NG> &o, const BlockHeader &hd,
+                                              const uint32_t *__restrict__ hdr, uint32_t blk,
+                                              const float *__restrict__ vals, const float *__restrict__ B,
+                                              uint32_t N, uint32_t col0, uint32_t lane)
+{
+    typedef typename Vec<VEC>::type V;
+    const uint32_t g = lane >> 4;
+    // columns of the g-th active column of bricks 0..3 (one 16-byte load per lane)
+    const uint4 c4 = reinterpret_cast<const uint4 *>(hdr + size_t(blk) * kHdrWords)[g];
+    const uint32_t cols[4] = {c4.x, c4.y, c4.z, c4.w};
+    o.live = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint64_t bm = hd.bitmap[j];
+        if (bm == 0) continue;                    // wave-uniform: bricks made of padding only
+        o.live |= 1ull << j;
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
+        o.a[j] = ((bm >> lane) & 1ull) ? vals[hd.voff[j] + below] : 0.0f;
+        const float *brow = B + size_t(cols[j]) * N;
+#pragma unroll
+        for (int ng = 0; ng < NG; ++ng) {
+            const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
+            if (c < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + c);
+            else o.b[j][ng] = V(0.0f);
+        }
+    }
+}
+
+template <int VEC, int NG>
+__device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x4 (&acc)[NG][VEC])
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (!((o.live >> j) & 1ull)) continue;
+#pragma unroll
+        for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[j], vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
+    }
+}
+
+// chunks[i] = {first block, end block, row panel, atomic}.  A work item is (chunk, slab);
+// slab s covers columns [s*16*VEC*NG, (s+1)*16*VEC*NG).  Lane L = 16*g + j owns, inside
+// column group ng, the VEC consecutive columns starting at s*slab + ng*16*VEC + j*VEC;
+// MFMA tile v of that group therefore holds the columns {.. + j*VEC + v}, and after the
+// MFMA lane L holds rows 4g..4g+3 of exactly those VEC columns -> one vector store per row.
+template <int VEC, int NG>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
+    const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
+    float *__restrict__ C, uint32_t N)
+{
+    typedef typename Vec<VEC>::type V;
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const uint32_t group = xcd_contiguous_id(blockIdx.x, groups_per_xcd);
+    const uint64_t item = uint64_t(group) * kWavesPerGroup + wave;
+    if (item >= uint64_t(num_chunks) * num_slabs) return;
+    const uint32_t chunk = uint32_t(item / num_slabs);
+    const uint32_t slab = uint32_t(item % num_slabs);
+    const uint4 ck = chunks[chunk];
+    const uint32_t start = __builtin_amdgcn_readfirstlane(ck.x);
+    const uint32_t end = __builtin_amdgcn_readfirstlane(ck.y);
+    const uint32_t panel = __builtin_amdgcn_readfirstlane(ck.z);
+    const uint32_t atomic = __builtin_amdgcn_readfirstlane(ck.w);
+    const uint32_t col0 = slab * (16u * VEC * NG) + (lane & 15u) * VEC;
+
+    f32x4 acc[NG][VEC];
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
+
+    // three-stage software pipeline: header(blk+2) | operands(blk+1) | MFMA(blk)
+    BlockOperands<VEC, NG> cur, nxt;
+    BlockHeader h_next;
+    if (start < end) {
+        BlockHeader h0 = load_header(hdr, start);
+        load_operands<VEC, NG>(cur, h0, hdr, start, vals, B, N, col0, lane);
+        if (start + 1 < end) h_next = load_header(hdr, start + 1);
+    }
+    for (uint32_t blk = start; blk < end; ++blk) {
+        const bool more = blk + 1 < end;
+        if (more) load_operands<VEC, NG>(nxt, h_next, hdr, blk + 1, vals, B, N, col0, lane);
+        if (blk + 2 < end) h_next = load_header(hdr, blk + 2);
+        mfma_block<VEC, NG>(cur, acc);
+        if (more) cur = nxt;
+    }
+
+    const uint32_t row0 = panel * 16u + (lane >> 4) * 4u;
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng) {
+        const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
+        if (c >= N) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float *dst = C + size_t(row0 + r) * N + c;
+            if (atomic) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
+            } else {
+                V out;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
+                *reinterpret_cast<V *>(dst) = out;
+            }
+        }
+    }
+}
+
+// Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).
+__global__ void zero_panels(const uint32_t *__restrict__ panels, uint32_t count, float *__restrict__ C, uint32_t N)
+{
+    const uint32_t p = blockIdx.x;
+    if (p >= count) return;
+    float *base = C + size_t(panels[p]) * 16u * N;
+    for (uint32_t i = threadIdx.x; i < 16u * N; i += blockDim.x) base[i] = 0.0f;
+}
+
+// One group of L = 1<<LOG_L lanes per row; lane t of the group owns VEC consecutive columns
+// starting at slab*L*VEC + t*VEC.  Nonzeros are fetched L at a time, one per lane, then
+// broadcast one after the other, so each C element accumulates its row in storage order.
+// row_list == nullptr: rows 0..num_rows-1.
+template <int VEC, int LOG_L>
+__global__ __launch_bounds__(256) void csr_rows(const uint32_t *__restrict__ row_list, uint32_t num_rows,
+                                                uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+                                                const uint32_t *__restrict__ cols, const float *__restrict__ vals,
+                                                const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+{
+    typedef typename Vec<VEC>::type V;
+    constexpr uint32_t L = 1u << LOG_L;
+    const uint32_t t = threadIdx.x & (L - 1);
+    const uint64_t gid = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> LOG_L;
+    // whole groups leave together, so shuffles below never read a retired lane of the same group
+    if (gid >= uint64_t(num_rows) * num_slabs) return;
+    const uint32_t ridx = uint32_t(gid / num_slabs);
+    const uint32_t slab = uint32_t(gid % num_slabs);
+    const uint32_t row = row_list ? row_list[ridx] : ridx;
+    const uint32_t c0 = slab * L * VEC + t * VEC;
+    const bool live = c0 < N;
+    const uint32_t s = rowPtr[row], e = rowPtr[row + 1];
+    V acc = V(0.0f);
+    for (uint32_t base = s; base < e; base += L) {
+        const uint32_t mine = base + t;
+        uint32_t my_col = 0;
+        float my_val = 0.0f;
+        if (mine < e) { my_col = cols[mine]; my_val = vals[mine]; }
+        const uint32_t cnt = min(L, e - base);
+        for (uint32_t q = 0; q < cnt; ++q) {
+            const uint32_t c = __shfl(my_col, int(q), int(L));
+            const float a = __shfl(my_val, int(q), int(L));
+            if (live) {
+                const V b = *reinterpret_cast<const V *>(B + size_t(c) * N + c0);
+                acc += a * b;
+            }
+        }
+    }
+    if (live) *reinterpret_cast<V *>(C + size_t(row) * N + c0) = acc;
+}
+
+// Thread per C element (inc/SPMM.cuh:898-920 restated for fp32 and a 64x4 thread tile).
+__global__ __launch_bounds__(256) void csr_thread_per_element(const uint32_t *__restrict__ rowPtr,
+                                                              const uint32_t *__restrict__ cols,
+                                                              const float *__restrict__ vals,
+                                                              const float *__restrict__ B, float *__restrict__ C,
+                                                              uint32_t M, uint32_t N)
+{
+    const uint32_t col = blockIdx.x * 64u + threadIdx.x;
+    const uint32_t row = blockIdx.y * 4u + threadIdx.y;
+    if (row >= M || col >= N) return;
+    float sum = 0.0f;
+    for (uint32_t i = rowPtr[row]; i < rowPtr[row + 1]; ++i) sum += vals[i] * B[size_t(cols[i]) * N + col];
+    C[size_t(row) * N + col] = sum;
+}
+
+// Wavefront per row, lane L handles columns L, L+64, ...; every lane reads (col, val) itself.
+__global__ __launch_bounds__(256) void csr_wave_scalar(const uint32_t *__restrict__ rowPtr,
+                                                       const uint32_t *__restrict__ cols,
+                                                       const float *__restrict__ vals, const float *__restrict__ B,
+                                                       float *__restrict__ C, uint32_t M, uint32_t N)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t row = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+    if (row >= M) return;
+    const uint32_t s = rowPtr[row], e = rowPtr[row + 1];
+    for (uint32_t c = lane; c < N; c += 64u) {
+        float sum = 0.0f;
+        for (uint32_t i = s; i < e; ++i) sum += vals[i] * B[size_t(cols[i]) * N + c];
+        C[row * N + c] = sum;
+    }
+}
+
+}  // namespace cute_dev

@@ -1,0 +1,249 @@
+/*
+ * cutespmm.h -- C ABI of the MI355X (gfx950) brick-blocked SpMM library, libcutespmm.so.
+ *
+ * C = A * B with A sparse fp32 (hybrid row-panel brick format, "HRPB"), B and C dense
+ * fp32 row-major.  Every entry point takes plain pointers and sizes.  Functions in the
+ * "host" groups never touch the GPU; functions in the "device" groups need one.
+ *
+ * Each declaration cites the reference interface it stands in for (paths relative to
+ * the reference tree).  All functions returning int return CUTE_OK (0) or a negative
+ * cute_status; cute_status_string() names it.  No function calls exit().
+ *
+ * Threading: handles are thread-compatible (use one plan per host thread); there is no
+ * hidden global state apart from a lazily created per-process device context.
+ */
+#ifndef CUTESPMM_H
+#define CUTESPMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Canonical format constants (inc.h:16-37 with the shipped -DTM=16 -DTK=16). */
+#define CUTE_TM 16u              /* rows per row panel                                  */
+#define CUTE_TK 16u              /* active columns per block                            */
+#define CUTE_BRICK_M 16u         /* brick = 16 rows x 4 active columns                  */
+#define CUTE_BRICK_K 4u
+#define CUTE_META_WORDS 36u      /* MetaDataSize, inc.h:36                              */
+#define CUTE_CHUNK_WORDS 128u    /* block records are padded to 512-byte chunks         */
+#define CUTE_TILED_HDR_WORDS 32u /* one 128-byte header line per block, device layout   */
+
+typedef enum cute_status {
+    CUTE_OK = 0,
+    CUTE_ERR_IO = -1,          /* file missing / unreadable / malformed                   */
+    CUTE_ERR_SHAPE = -2,       /* M or K not a multiple of 16, N == 0, size overflow      */
+    CUTE_ERR_UNSORTED = -3,    /* a CSR row has unsorted or duplicate columns             */
+    CUTE_ERR_RANGE = -4,       /* an index is out of range                                */
+    CUTE_ERR_ARG = -5,         /* null pointer / bad enum                                 */
+    CUTE_ERR_NOMEM = -6,
+    CUTE_ERR_HIP = -7,         /* a HIP runtime call failed; see cute_last_hip_error()    */
+    CUTE_ERR_NO_DEVICE = -8,   /* no gfx950 device visible                                */
+    CUTE_ERR_FORMAT = -9       /* a format stream failed validation                       */
+} cute_status;
+
+const char *cute_status_string(int status);
+/* hipGetErrorString of the most recent failing HIP call on this thread (""), never NULL. */
+const char *cute_last_hip_error(void);
+void cute_free(void *p);       /* releases any array returned by this library            */
+
+/* ------------------------------------------------------------------------------------
+ * host: MatrixMarket -> CSR.                       Replaces MTX_READER (IO.cu:2-88).
+ * M and K are rounded up to multiples of 16 (IO.cu:30-31); symmetric files are mirrored
+ * (IO.cu:42-44,77-84); entries stay in file order inside a row (IO.cu:71-75).
+ * keep_values == 0 reproduces the reference (every value 1.0f, IO.cu:68,81);
+ * keep_values != 0 parses the third token (1.0 for pattern files).
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_csr {
+    uint32_t M, K, nnz;
+    uint32_t *rowPtr;          /* [M+1]                                                    */
+    uint32_t *cols;            /* [nnz]                                                    */
+    float *vals;               /* [nnz]                                                    */
+} cute_csr;
+
+int cute_mtx_read(const char *path, int keep_values, cute_csr *out);
+void cute_csr_release(cute_csr *csr);
+/* Sorts every row by column (stable w.r.t. values) so that it satisfies the HRPB
+ * precondition; returns CUTE_ERR_UNSORTED if a row holds a duplicate column. */
+int cute_csr_sort_rows(cute_csr *csr);
+
+/* ------------------------------------------------------------------------------------
+ * host: CSR -> canonical HRPB.          Replaces HRPB::HRPB + DATASTRUCT (data.cu:80-335).
+ * Output arrays are word-for-word those of the reference (record layout inc.h:28-37,
+ * written at data.cu:212-296).  The CSR arrays are borrowed, as in data.cu:82-84, and
+ * must outlive the object.  Preconditions are checked, not assumed: M,K multiples of 16,
+ * columns strictly increasing inside each row and < K.
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_hrpb_host {
+    uint32_t M, K;
+    uint32_t numRowPanels;     /* M / 16                                                   */
+    uint32_t numBlocks;        /* blockedRowPtr[numRowPanels]                              */
+    uint64_t numWords;         /* length of blocksData                                     */
+    uint32_t *blockedRowPtr;   /* [numRowPanels+1]                                         */
+    uint32_t *activeCols;      /* [numBlocks*16]                                           */
+    uint64_t *sizePtr;         /* [numBlocks+1]                                            */
+    uint32_t *blocksData;      /* [numWords]                                               */
+    const uint32_t *rowPtr;    /* borrowed CSR                                             */
+    const uint32_t *cols;
+    const float *vals;
+    uint32_t nnz;
+    uint32_t numBricks;        /* non-empty 16x4 bricks                                    */
+} cute_hrpb_host;
+
+int cute_hrpb_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols,
+                    const float *vals, cute_hrpb_host *out);
+void cute_hrpb_host_release(cute_hrpb_host *h);
+
+/* ------------------------------------------------------------------------------------
+ * host: canonical HRPB <-> MFMA-tiled device layout (no reference counterpart for the
+ * layout itself; it re-tiles what kernel.cu:16-29 decodes per lane).  Per block one
+ * 128-byte header line:
+ *   words  0..15  active columns, word k*4+j = column of brick j, k-th column in brick
+ *   words 16..23  four 64-bit bitmaps, bit k*16+row  <=> canonical bit row*4+k, so that
+ *                 bit L is the A operand of wavefront lane L in v_mfma_f32_16x16x4_f32
+ *   words 24..27  index into vals[] of each brick's first value
+ *   word  28      nonzeros in the block;  words 29..31 zero
+ * vals[] holds every brick's nonzeros in bitmap (lane) order.  cute_hrpb_untile()
+ * inverts the mapping exactly; the pair is a bijection on valid streams.
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_hrpb_tiled {
+    uint32_t M, K, numRowPanels, numBlocks;
+    uint64_t numVals;
+    uint32_t *blockedRowPtr;   /* [numRowPanels+1] copy                                    */
+    uint32_t *hdr;             /* [numBlocks*32]                                           */
+    float *vals;               /* [numVals]                                                */
+} cute_hrpb_tiled;
+
+int cute_hrpb_retile(const cute_hrpb_host *h, cute_hrpb_tiled *out);
+int cute_hrpb_untile(const cute_hrpb_tiled *t, cute_hrpb_host *out);
+void cute_hrpb_tiled_release(cute_hrpb_tiled *t);
+
+/* ------------------------------------------------------------------------------------
+ * host: launch partition.            Replaces SPMM_TC::partition (spmm.cu:776-812).
+ * Same arithmetic; the machine enters through `slots` (work items resident on the whole
+ * device; num_sms*num_thread_blocks at spmm.cu:778-779) and `nbN` (work items along N).
+ * out4 receives {first block, end block, panel, atomic} quadruples; returns their count
+ * (which may exceed cap: call again with a larger buffer), or a negative status.
+ * ---------------------------------------------------------------------------------- */
+int64_t cute_partition(uint32_t numRowPanels, const uint32_t *blockedRowPtr, uint32_t nbN,
+                       uint32_t slots, uint32_t *out4, uint64_t cap);
+
+/* ------------------------------------------------------------------------------------
+ * host: result comparison.   Replaces check_gemm_correctness_coo (inc.h:84-109):
+ * max over i with C_ref[i] != 0 of |C_ref[i]-C_test[i]| / |C_ref[i]|.
+ * cute_backward_error() is the cancellation-robust companion:
+ * max_ij |C_ref-C_test|_ij / sum_k |a_ik||b_kj| (0/0 counts as 0).
+ * ---------------------------------------------------------------------------------- */
+float cute_check_gemm_correctness(const float *C_ref, const float *C_test, uint32_t M, uint32_t N);
+float cute_backward_error(const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
+                          const float *B, const float *C_ref, const float *C_test,
+                          uint32_t M, uint32_t N);
+
+/* ------------------------------------------------------------------------------------
+ * host: seeded synthetic inputs (the reference only reads .mtx files; run.cu:24-27 fills
+ * B with rand()).  Counter-based generator, so values do not depend on thread count.
+ *   kind 1 uniform:  M x M, `p0` distinct uniformly random columns per row, values U(-1,1)
+ *   kind 2 stencil:  9-point stencil on a p0 x p0 grid, 8 on / -1 off the diagonal + U(-.01,.01)
+ *   kind 3 fem:      p0 node blocks of 6x6, diagonal + ~9 neighbours within +-p1 blocks, symmetric
+ *   kind 4 rmat:     2^p0 nodes, p1 edges per node, (.57,.19,.19,.05), symmetrised, +I, 1/sqrt(di dj)
+ *   kind 5 banded:   M = p0 rows, p1 distinct columns per row within +-p2 of the diagonal, U(-1,1)
+ * Rows come out sorted by column; M is a multiple of 16 for the stock parameters.
+ * ---------------------------------------------------------------------------------- */
+int cute_gen_matrix(int kind, uint64_t seed, uint32_t p0, uint32_t p1, uint32_t p2, cute_csr *out);
+/* dist 0: U(0,1)   1: U(-1,1)   2: N(0,1) (Box-Muller).  Element i depends only on (seed, i). */
+int cute_gen_dense(uint64_t seed, int dist, uint64_t count, float *out);
+
+/* ------------------------------------------------------------------------------------
+ * device: upload.        Replaces the cudaMalloc/cudaMemcpy tail of DATASTRUCT
+ * (data.cu:327-334) and HRPB::freeDevice (data.cu:336-339).  Uploads the MFMA-tiled
+ * layout, the per-panel descriptors and the borrowed CSR (for the sparse-panel path).
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_hrpb_dev cute_hrpb_dev;
+int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out);
+void cute_hrpb_dev_free(cute_hrpb_dev *d);
+uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d); /* device bytes held */
+
+/* ------------------------------------------------------------------------------------
+ * device: plan + launch.   Replaces SPMM_TC::SPMM_TC / initialize_conditions / partition
+ * (spmm.cu:276-822) and SPMM_TC::run (spmm.cu:823-839).
+ * ---------------------------------------------------------------------------------- */
+typedef enum cute_path {
+    CUTE_PATH_AUTO = 0,        /* per-panel choice between brick and row kernels          */
+    CUTE_PATH_BRICK = 1,       /* every panel through the MFMA brick kernel               */
+    CUTE_PATH_ROWS = 2         /* every panel through the wavefront-per-row kernel        */
+} cute_path;
+
+typedef enum cute_precision {
+    CUTE_PREC_FP32 = 0,        /* v_mfma_f32_16x16x4_f32, fp32 operands                   */
+    CUTE_PREC_BF16X3 = 1       /* bf16 hi/lo split, three bf16 MFMA products              */
+} cute_precision;
+
+typedef struct cute_tunables {
+    int32_t path;              /* cute_path                                               */
+    int32_t precision;         /* cute_precision                                          */
+    float min_reuse;           /* AUTO: panels with nnz/activeCols below this go to ROWS; <=0: default */
+    uint32_t slots;            /* resident work items assumed by the partition; 0: derive from device */
+    uint32_t max_chunk_blocks; /* upper bound on blocks per work item; 0: none            */
+    uint32_t brick_groups;     /* 16-lane column groups per lane in the brick kernel (1 or 2); 0: default */
+    uint32_t reserved[2];
+} cute_tunables;
+
+typedef struct cute_plan_info {
+    uint32_t N;
+    uint32_t slabWidth;        /* columns of C per work item                              */
+    uint32_t numSlabs;
+    uint32_t numChunks;        /* brick-kernel work items along the panel axis            */
+    uint32_t numAtomicChunks;  /* of which combine through atomics                        */
+    uint32_t numBrickPanels, numRowPanelsSparse, numEmptyPanels;
+    uint32_t slots;
+    uint32_t precision, path;
+    uint32_t reserved[5];
+} cute_plan_info;
+
+typedef struct cute_spmm_plan cute_spmm_plan;
+int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunables *t /* may be NULL */,
+                          cute_spmm_plan **out);
+int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out);
+void cute_spmm_plan_free(cute_spmm_plan *p);
+/* dB [K x N], dC [M x N]: device pointers, row-major, 16-byte aligned.  Asynchronous on
+ * `stream` (a hipStream_t, NULL = default stream).  C is fully overwritten: the caller
+ * need not zero it (the reference requires cudaMemset first, run.cu:43,49). */
+int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * device: plain CSR SpMM kernels -- the fp32 CSR comparison path.  Replaces
+ * GPU_CSR_cuSPARSE_NEW (spmm.cu:860-960); the three algorithms restate the simple kernels
+ * of inc/SPMM.cuh (898-920 thread per element, 1061-1146 wavefront per row) and a
+ * vectorised wavefront-per-row variant.
+ *   alg 0: thread per (row, column)   1: wavefront per row, scalar lanes
+ *   alg 2: wavefront per row, float4/float2 lanes
+ * cute_csr_spmm_dev takes device pointers; cute_gpu_csr_spmm takes host pointers, copies,
+ * runs one warm-up plus `iters` timed launches and returns ms per launch (< 0: -status).
+ * ---------------------------------------------------------------------------------- */
+int cute_csr_spmm_dev(int alg, const uint32_t *dRowPtr, const uint32_t *dCols, const float *dVals,
+                      const float *dB, float *dC, uint32_t M, uint32_t N, void *stream);
+float cute_gpu_csr_spmm(const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t nnz,
+                        const float *hB, float *hC, uint32_t m, uint32_t k, uint32_t n, int iters, int alg);
+
+/* device pointers of the uploaded CSR copy (for cute_csr_spmm_dev on the same matrix). */
+int cute_hrpb_dev_csr(const cute_hrpb_dev *d, const uint32_t **dRowPtr, const uint32_t **dCols,
+                      const float **dVals);
+
+/* ------------------------------------------------------------------------------------
+ * device: timing helper used by the drivers.  Runs `warmup` untimed and `iters` timed
+ * launches of the plan on `stream`, each bracketed by HIP events on that stream; writes
+ * per-launch milliseconds to ms_out[iters].
+ * ---------------------------------------------------------------------------------- */
+int cute_spmm_time(cute_spmm_plan *p, const float *dB, float *dC, void *stream, int warmup, int iters,
+                   float *ms_out);
+int cute_csr_spmm_time(int alg, const cute_hrpb_dev *d, const float *dB, float *dC, uint32_t N,
+                       void *stream, int warmup, int iters, float *ms_out);
+
+int cute_device_info(int *num_cus, int *wave_size, char *arch_name, size_t arch_cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUTESPMM_H */

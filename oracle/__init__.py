@@ -1,0 +1,133 @@
+"""ctypes/numpy front end of the CPU oracle (``cute_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: importable from ``tests/``, the smoke check and the
+benchmark's CPU-baseline leg.  The shipped package never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libcute_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile ``cute_oracle.c`` with the Makefile beside it."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_partition.restype = C.c_uint32
+        _lib.orc_check_gemm.restype = C.c_float
+        _lib.orc_free.argtypes = [C.c_void_p]
+    return _lib
+
+
+def _p(a, t):
+    return a.ctypes.data_as(C.POINTER(t))
+
+
+def _take(ptr, n, dtype):
+    """Copy n items from a malloc'ed pointer into a numpy array and free it."""
+    out = np.ctypeslib.as_array(ptr, shape=(max(int(n), 1),)).astype(dtype, copy=True)[: int(n)]
+    lib().orc_free(C.cast(ptr, C.c_void_p))
+    return out
+
+
+def mtx_read(path):
+    """IO.cu:10-87 -> (M, K, nnz, rowPtr, cols, vals)."""
+    M, K, nnz = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    rp, cl, vl = C.POINTER(C.c_uint32)(), C.POINTER(C.c_uint32)(), C.POINTER(C.c_float)()
+    rc = lib().orc_mtx_read(os.fsencode(path), C.byref(M), C.byref(K), C.byref(nnz),
+                            C.byref(rp), C.byref(cl), C.byref(vl))
+    if rc:
+        raise IOError("orc_mtx_read(%s) failed: %d" % (path, rc))
+    total = rp[M.value]
+    return (M.value, K.value, nnz.value, _take(rp, M.value + 1, np.uint32),
+            _take(cl, total, np.uint32), _take(vl, total, np.float32))
+
+
+def hrpb_build(M, K, rowPtr, cols, vals):
+    """data.cu:94-335 -> dict of the four canonical arrays."""
+    rowPtr = np.ascontiguousarray(rowPtr, np.uint32)
+    cols = np.ascontiguousarray(cols, np.uint32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    brp, ac, bd = (C.POINTER(C.c_uint32)() for _ in range(3))
+    sp = C.POINTER(C.c_uint64)()
+    nb, nw = C.c_uint32(), C.c_uint64()
+    rc = lib().orc_hrpb_build(C.c_uint32(M), C.c_uint32(K), _p(rowPtr, C.c_uint32), _p(cols, C.c_uint32),
+                              _p(vals, C.c_float), C.byref(brp), C.byref(ac), C.byref(sp), C.byref(bd),
+                              C.byref(nb), C.byref(nw))
+    if rc:
+        raise ValueError("orc_hrpb_build failed: %d" % rc)
+    P = M // 16
+    return dict(M=M, K=K, numRowPanels=P, numBlocks=nb.value, numWords=nw.value,
+                blockedRowPtr=_take(brp, P + 1, np.uint32),
+                activeCols=_take(ac, nb.value * 16, np.uint32),
+                sizePtr=_take(sp, nb.value + 1, np.uint64),
+                blocksData=_take(bd, nw.value, np.uint32))
+
+
+def partition(blockedRowPtr, nbN, slots):
+    """spmm.cu:776-812 -> uint32 array [n,4] of {start,end,panel,atomic}."""
+    brp = np.ascontiguousarray(blockedRowPtr, np.uint32)
+    P = len(brp) - 1
+    cap = int(brp[-1]) + P + 1
+    out = np.zeros((cap, 4), np.uint32)
+    n = lib().orc_partition(C.c_uint32(P), _p(brp, C.c_uint32), C.c_uint32(nbN), C.c_uint32(slots),
+                            _p(out, C.c_uint32), C.c_uint32(cap))
+    assert n <= cap
+    return out[:n].copy()
+
+
+def spmm_coo(rows, cols, vals, B, M):
+    rows = np.ascontiguousarray(rows, np.uint32)
+    cols = np.ascontiguousarray(cols, np.uint32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    B = np.ascontiguousarray(B, np.float32)
+    K, N = B.shape
+    Cm = np.empty((M, N), np.float32)
+    lib().orc_spmm_coo(_p(rows, C.c_uint32), _p(cols, C.c_uint32), _p(vals, C.c_float), _p(B, C.c_float),
+                       _p(Cm, C.c_float), C.c_uint32(M), C.c_uint32(K), C.c_uint32(N), C.c_uint32(len(vals)))
+    return Cm
+
+
+def spmm_csr(rowPtr, cols, vals, B, out=None):
+    rowPtr = np.ascontiguousarray(rowPtr, np.uint32)
+    cols = np.ascontiguousarray(cols, np.uint32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    B = np.ascontiguousarray(B, np.float32)
+    M, N = len(rowPtr) - 1, B.shape[1]
+    Cm = np.empty((M, N), np.float32) if out is None else out
+    lib().orc_spmm_csr(_p(rowPtr, C.c_uint32), _p(cols, C.c_uint32), _p(vals, C.c_float), _p(B, C.c_float),
+                       _p(Cm, C.c_float), C.c_uint32(M), C.c_uint32(N))
+    return Cm
+
+
+def spmm_hrpb(h, B):
+    B = np.ascontiguousarray(B, np.float32)
+    N = B.shape[1]
+    Cm = np.empty((h["M"], N), np.float32)
+    lib().orc_spmm_hrpb(C.c_uint32(h["M"]), C.c_uint32(N), _p(h["blockedRowPtr"], C.c_uint32),
+                        _p(h["activeCols"], C.c_uint32), _p(h["sizePtr"], C.c_uint64),
+                        _p(h["blocksData"], C.c_uint32), _p(B, C.c_float), _p(Cm, C.c_float))
+    return Cm
+
+
+def check_gemm(C_ref, C_test):
+    """inc.h:84-109; the first argument is the trusted result."""
+    a = np.ascontiguousarray(C_ref, np.float32)
+    b = np.ascontiguousarray(C_test, np.float32)
+    assert a.shape == b.shape
+    M, N = a.shape
+    return float(lib().orc_check_gemm(_p(a, C.c_float), _p(b, C.c_float), C.c_uint32(M), C.c_uint32(N)))
