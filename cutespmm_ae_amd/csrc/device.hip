@@ -158,7 +158,13 @@ int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
         d->panelCols[p] = live;
     }
     rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
-    if (rc == CUTE_OK) rc = upload(&d->dVals, t.vals, t.numVals);
+    if (rc == CUTE_OK) {
+        // one wavefront of zero padding behind the values: the brick kernel loads A operands
+        // unconditionally at (brick offset + lane rank)
+        std::vector<float> padded(t.numVals + 64, 0.0f);
+        if (t.numVals) std::memcpy(padded.data(), t.vals, t.numVals * sizeof(float));
+        rc = upload(&d->dVals, padded.data(), padded.size());
+    }
     if (rc == CUTE_OK) rc = upload(&d->dRowPtr, h->rowPtr, uint64_t(h->M) + 1);
     if (rc == CUTE_OK) rc = upload(&d->dCols, h->cols, h->nnz);
     if (rc == CUTE_OK) rc = upload(&d->dCsrVals, h->vals, h->nnz);
@@ -244,14 +250,39 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         if (nblk) (rows ? n_rows : n_brick)++;
     }
 
-    // chunk list for the brick kernel
-    const uint32_t slots = t.slots ? t.slots : uint32_t(c.num_cus) * 4u * 4u;   // 4 SIMDs x 4 wavefronts
+    // chunk list for the brick kernel.  With t.slots set, the reference arithmetic
+    // (spmm.cu:776-812) decides which panels are cut; its default there would cut every panel
+    // that is one block above the (floored) mean as soon as the device holds all work items
+    // at once, which is the normal case on 256 CUs.  The default policy therefore cuts only
+    // outliers: a panel is split when it is more than twice as long as the per-item share
+    // of the whole job (and at least 8 blocks), into pieces of about that share.
+    const uint32_t resident = uint32_t(c.num_cus) * 4u * 8u;   // 4 SIMDs x 8 wavefronts per CU
+    const uint32_t slots = t.slots ? t.slots : resident;
     std::vector<uint32_t> quads;
-    {
+    if (t.slots) {
         int64_t n = cute_partition(d->P, d->brp.data(), num_slabs, slots, nullptr, 0);
         if (n < 0) { delete p; return int(n); }
         quads.resize(uint64_t(n) * 4);
         cute_partition(d->P, d->brp.data(), num_slabs, slots, quads.data(), uint64_t(n));
+    } else {
+        uint64_t work = 0;
+        for (uint32_t q = 0; q < d->P; ++q)
+            if (!to_rows[q]) work += d->brp[q + 1] - d->brp[q];
+        const uint64_t mean = n_brick ? (work + n_brick - 1) / n_brick : 1;
+        const uint64_t share = (work * num_slabs + resident - 1) / resident;
+        const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, mean), 8));
+        for (uint32_t q = 0; q < d->P; ++q) {
+            const uint32_t s = d->brp[q], e = d->brp[q + 1];
+            if (s == e || to_rows[q]) continue;
+            const uint32_t nblk = e - s;
+            if (nblk <= 2 * target) {
+                quads.insert(quads.end(), {s, e, q, 0u});
+                continue;
+            }
+            const uint32_t pieces = (nblk + target - 1) / target;
+            const uint32_t step = (nblk + pieces - 1) / pieces;
+            for (uint32_t cs = s; cs < e; cs += step) quads.insert(quads.end(), {cs, std::min(e, cs + step), q, 1u});
+        }
     }
     std::vector<uint4> chunks;
     std::vector<uint32_t> atomic_panels;
@@ -301,15 +332,22 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
 namespace {
 
-template <int VEC, int NG>
-void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+template <int VEC, int NG, bool FULL>
+void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
 {
     const uint64_t items = uint64_t(p->info.numChunks) * p->info.numSlabs;
     const uint32_t groups = uint32_t((items + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup);
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
-    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG>), dim3(per_xcd * cute_dev::kNumXcd),
+    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
                        dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
                        p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+}
+
+template <int VEC, int NG>
+void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+{
+    if (p->info.N % p->info.slabWidth == 0) launch_brick_full<VEC, NG, true>(p, dB, dC, s);
+    else launch_brick_full<VEC, NG, false>(p, dB, dC, s);
 }
 
 template <int VEC>

@@ -39,22 +39,24 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t gro
     return (bid % kNumXcd) * groups_per_xcd + bid / kNumXcd;
 }
 
-struct BlockHeader {          // wave-uniform part of one 128-byte header line
-    uint64_t bitmap[4];
-    uint32_t voff[4];
+struct BlockHeader {          // one 128-byte header line as a wavefront sees it
+    uint64_t bitmap[4];       // wave-uniform (scalar loads)
+    uint32_t voff[4];         // wave-uniform
+    uint4 cols;               // per lane: the (lane/16)-th active column of bricks 0..3
 };
 
 template <int VEC, int NG>
 struct BlockOperands {
-    float a[4];                                   // A operand per brick (lane L <-> bitmap bit L)
+    float a[4];                                   // value at (brick offset + lane rank), before masking
+    uint64_t bitmap[4];                           // wave-uniform: lane L is a nonzero iff bit L
     typename Vec<VEC>::type b[4][NG];             // B operand vectors per brick and column group
-    uint64_t live;                                // bit j set: brick j is non-empty (wave-uniform)
 };
 
-__device__ __forceinline__ BlockHeader load_header(const uint32_t *__restrict__ hdr, uint32_t blk)
+__device__ __forceinline__ BlockHeader load_header(const uint32_t *__restrict__ hdr, uint32_t blk, uint32_t lane)
 {
     const uint32_t *h = hdr + size_t(blk) * kHdrWords;
     BlockHeader r;
+    r.cols = reinterpret_cast<const uint4 *>(h)[lane >> 4];
     const uint64_t *bm = reinterpret_cast<const uint64_t *>(h + 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j) r.bitmap[j] = bm[j];
@@ -63,46 +65,43 @@ __device__ __forceinline__ BlockHeader load_header(const uint32_t *__restrict__ 
     return r;
 }
 
-template <int VEC, int NG>
+// Issues every load of one block without a branch: bricks that consist of padding only
+// have an all-zero bitmap and padding columns point at B row 0, so they contribute
+// 0 * B[0][.] (B must be finite, as in the reference, kernel.cu:26-27,149).  vals[] is
+// padded by one wavefront of floats so that the unconditional A load never leaves it.
+template <int VEC, int NG, bool FULL>
 __device__ __forceinline__ void load_operands(BlockOperands<VEC, NG> &o, const BlockHeader &hd,
-                                              const uint32_t *__restrict__ hdr, uint32_t blk,
                                               const float *__restrict__ vals, const float *__restrict__ B,
                                               uint32_t N, uint32_t col0, uint32_t lane)
 {
     typedef typename Vec<VEC>::type V;
-    const uint32_t g = lane >> 4;
-    // columns of the g-th active column of bricks 0..3 (one 16-byte load per lane)
-    const uint4 c4 = reinterpret_cast<const uint4 *>(hdr + size_t(blk) * kHdrWords)[g];
-    const uint32_t cols[4] = {c4.x, c4.y, c4.z, c4.w};
-    o.live = 0;
+    const uint32_t cols[4] = {hd.cols.x, hd.cols.y, hd.cols.z, hd.cols.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint64_t bm = hd.bitmap[j];
-        if (bm == 0) continue;                    // wave-uniform: bricks made of padding only
-        o.live |= 1ull << j;
         const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
-        o.a[j] = ((bm >> lane) & 1ull) ? vals[hd.voff[j] + below] : 0.0f;
-        const float *brow = B + size_t(cols[j]) * N;
+        o.a[j] = vals[hd.voff[j] + below];       // masked when consumed, so nothing waits here
+        o.bitmap[j] = bm;
+        const float *brow = B + size_t(cols[j]) * N + col0;
 #pragma unroll
         for (int ng = 0; ng < NG; ++ng) {
-            const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
-            if (c < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + c);
+            if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + ng * 16 * VEC);
             else o.b[j][ng] = V(0.0f);
         }
     }
 }
 
 template <int VEC, int NG>
-__device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x4 (&acc)[NG][VEC])
+__device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x4 (&acc)[NG][VEC], uint32_t lane)
 {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        if (!((o.live >> j) & 1ull)) continue;
+        const float a = ((o.bitmap[j] >> lane) & 1ull) ? o.a[j] : 0.0f;
 #pragma unroll
         for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-                acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[j], vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
+                acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
     }
 }
 
@@ -111,7 +110,8 @@ __device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x
 // column group ng, the VEC consecutive columns starting at s*slab + ng*16*VEC + j*VEC;
 // MFMA tile v of that group therefore holds the columns {.. + j*VEC + v}, and after the
 // MFMA lane L holds rows 4g..4g+3 of exactly those VEC columns -> one vector store per row.
-template <int VEC, int NG>
+// FULL: N is a multiple of the slab width, so no column guard is compiled in.
+template <int VEC, int NG, bool FULL>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
     const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
@@ -138,27 +138,64 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
 
-    // three-stage software pipeline: header(blk+2) | operands(blk+1) | MFMA(blk)
-    BlockOperands<VEC, NG> cur, nxt;
-    BlockHeader h_next;
-    if (start < end) {
-        BlockHeader h0 = load_header(hdr, start);
-        load_operands<VEC, NG>(cur, h0, hdr, start, vals, B, N, col0, lane);
-        if (start + 1 < end) h_next = load_header(hdr, start + 1);
+    // Software pipeline, unrolled by two so that the operand sets ping-pong without copies:
+    // header lines run two blocks ahead of the MFMAs, operand loads one block ahead.  The
+    // steady-state loop is a single basic block (every prefetch in it is in range), so the
+    // scheduling barriers really keep each load group ahead of the MFMAs that hide it.
+    BlockOperands<VEC, NG> opA, opB;
+    BlockHeader hd, hn;
+    uint32_t blk = start;
+    if (blk < end) {
+        hd = load_header(hdr, blk, lane);
+        if (blk + 1 < end) hn = load_header(hdr, blk + 1, lane);
+        load_operands<VEC, NG, FULL>(opA, hd, vals, B, N, col0, lane);
+        hd = hn;
     }
-    for (uint32_t blk = start; blk < end; ++blk) {
-        const bool more = blk + 1 < end;
-        if (more) load_operands<VEC, NG>(nxt, h_next, hdr, blk + 1, vals, B, N, col0, lane);
-        if (blk + 2 < end) h_next = load_header(hdr, blk + 2);
-        mfma_block<VEC, NG>(cur, acc);
-        if (more) cur = nxt;
+    // Inside a stage the next header line is requested before the operand loads: loads
+    // return in order, so the later wait for that header then leaves the operand loads in flight.
+    while (blk + 4 <= end) {          // opA holds block blk, hd the header of blk+1
+        hn = load_header(hdr, blk + 2, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        load_operands<VEC, NG, FULL>(opB, hd, vals, B, N, col0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opA, acc, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        hd = load_header(hdr, blk + 3, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        load_operands<VEC, NG, FULL>(opA, hn, vals, B, N, col0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opB, acc, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        blk += 2;
+    }
+    const uint32_t rem = end - blk;   // 0 (empty chunk), 1, 2 or 3 blocks left; opA/hd as above
+    if (rem == 1) {
+        mfma_block<VEC, NG>(opA, acc, lane);
+    } else if (rem == 2) {
+        load_operands<VEC, NG, FULL>(opB, hd, vals, B, N, col0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opA, acc, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opB, acc, lane);
+    } else if (rem == 3) {
+        hn = load_header(hdr, blk + 2, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        load_operands<VEC, NG, FULL>(opB, hd, vals, B, N, col0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opA, acc, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        load_operands<VEC, NG, FULL>(opA, hn, vals, B, N, col0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opB, acc, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block<VEC, NG>(opA, acc, lane);
     }
 
     const uint32_t row0 = panel * 16u + (lane >> 4) * 4u;
 #pragma unroll
     for (int ng = 0; ng < NG; ++ng) {
         const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
-        if (c >= N) continue;
+        if (!FULL && c >= N) continue;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             float *dst = C + size_t(row0 + r) * N + c;
