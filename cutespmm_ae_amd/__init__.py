@@ -85,6 +85,13 @@ def load_library():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise CuteError(-8, "libcutespmm.so is not built (run python -m cutespmm_ae_amd.build); no fallback path")
+    # torch carries its own copy of the HIP runtime.  Importing it first makes the dynamic
+    # loader bind this library to that same copy (matching SONAME); loaded the other way
+    # round the process would hold two HIP runtimes and the second one finds no device.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     lib.cute_status_string.restype = C.c_char_p
     lib.cute_status_string.argtypes = [C.c_int]
@@ -155,11 +162,18 @@ def _ptr(a, t):
     return a.ctypes.data_as(t)
 
 
-def _view(ptr, n, dtype):
+class _Owned(np.ndarray):
+    """ndarray view of library-owned memory that keeps its owner object alive."""
+    _owner = None
+
+
+def _view(ptr, n, dtype, owner=None):
     n = int(n)
     if n == 0:
         return np.zeros(0, dtype)
-    return np.ctypeslib.as_array(ptr, shape=(n,)).view(dtype)
+    a = np.ctypeslib.as_array(ptr, shape=(n,)).view(dtype).view(_Owned)
+    a._owner = owner
+    return a
 
 
 # --------------------------------------------------------------------------------------
@@ -171,17 +185,33 @@ class CSR:
     def __init__(self, raw):
         self._raw = raw
         self.M, self.K, self.nnz = raw.M, raw.K, raw.nnz
-        self.rowPtr = _view(raw.rowPtr, raw.M + 1, np.uint32)
-        self.cols = _view(raw.cols, raw.nnz, np.uint32)
-        self.vals = _view(raw.vals, raw.nnz, np.float32)
+        self._attach()
+
+    def _attach(self):
+        raw = self._raw
+        self.rowPtr = _view(raw.rowPtr, raw.M + 1, np.uint32, self._keep)
+        self.cols = _view(raw.cols, raw.nnz, np.uint32, self._keep)
+        self.vals = _view(raw.vals, raw.nnz, np.float32, self._keep)
+
+    @property
+    def _keep(self):
+        # the arrays outlive this wrapper if somebody still holds a view of them
+        if not hasattr(self, "_guard"):
+            self._guard = _CsrGuard(self._raw)
+        return self._guard
 
     def sort_rows(self):
         _check(load_library().cute_csr_sort_rows(C.byref(self._raw)), "cute_csr_sort_rows")
         return self
 
+
+class _CsrGuard:
+    def __init__(self, raw):
+        self.raw = raw
+
     def __del__(self):
         try:
-            load_library().cute_csr_release(C.byref(self._raw))
+            load_library().cute_csr_release(C.byref(self.raw))
         except Exception:
             pass
 
@@ -259,10 +289,11 @@ class HRPB:
         self.M, self.K = r.M, r.K
         self.numRowPanels, self.numBlocks, self.numWords = r.numRowPanels, r.numBlocks, r.numWords
         self.num_bricks, self.numNNZ = r.numBricks, r.nnz
-        self.blockedRowPtr = _view(r.blockedRowPtr, r.numRowPanels + 1, np.uint32)
-        self.activeCols = _view(r.activeCols, r.numBlocks * 16, np.uint32)
-        self.sizePtr = _view(r.sizePtr, r.numBlocks + 1, np.uint64)
-        self.blocksData = _view(r.blocksData, r.numWords, np.uint32)
+        self._guard = _HrpbGuard(r, self._dev)
+        self.blockedRowPtr = _view(r.blockedRowPtr, r.numRowPanels + 1, np.uint32, self._guard)
+        self.activeCols = _view(r.activeCols, r.numBlocks * 16, np.uint32, self._guard)
+        self.sizePtr = _view(r.sizePtr, r.numBlocks + 1, np.uint64, self._guard)
+        self.blocksData = _view(r.blocksData, r.numWords, np.uint32, self._guard)
 
     def as_dict(self):
         return dict(M=self.M, K=self.K, numRowPanels=self.numRowPanels, numBlocks=self.numBlocks,
@@ -307,12 +338,22 @@ class HRPB:
     def freeDevice(self):
         if self._dev:
             load_library().cute_hrpb_dev_free(self._dev)
-            self._dev = C.c_void_p()
+            self._dev.value = None
+
+
+class _HrpbGuard:
+    """Releases the host arrays and the device twin once the HRPB object and every view
+    of its arrays are gone (the CSR arrays it borrows are numpy-owned and kept by HRPB)."""
+
+    def __init__(self, raw, dev):
+        self.raw, self.dev = raw, dev
 
     def __del__(self):
         try:
-            self.freeDevice()
-            load_library().cute_hrpb_host_release(C.byref(self._raw))
+            lib = load_library()
+            if self.dev:
+                lib.cute_hrpb_dev_free(self.dev)
+            lib.cute_hrpb_host_release(C.byref(self.raw))
         except Exception:
             pass
 

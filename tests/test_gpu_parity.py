@@ -1,0 +1,230 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the
+same seeded inputs.
+
+Tolerances (fp32 MFMA / fp32 FMA paths):
+  * componentwise backward error  max |dC_ij| / sum_k |a_ik||b_kj|  <= 2e-6
+    (a row with n nonzeros summed in any order in fp32 is within n * 2^-24 of exact);
+  * the reference's own metric (inc.h:84-109), max relative error over non-zero reference
+    entries, <= 1e-5 on inputs without cancellation (A = 1, B in [0,1), the only regime the
+    reference ever evaluated it in, run.cu:24-27 + IO.cu:68);
+  * exact equality where every product and partial sum is exactly representable.
+"""
+import numpy as np
+import pytest
+
+from helpers import csr_from_dense, random_csr
+
+pytestmark = pytest.mark.gpu
+
+BERR = 2e-6
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch
+
+
+def _run(cs, torch, h, B, **kw):
+    N = B.shape[1]
+    dB = torch.from_numpy(np.ascontiguousarray(B)).cuda()
+    dC = torch.full((h.M, N), float("nan"), device="cuda")      # every element must be written
+    plan = cs.SPMM_TC(h, N, **kw)
+    plan.run(dB, dC)
+    torch.cuda.synchronize()
+    return dC.cpu().numpy(), plan
+
+
+def _paths(cs):
+    return [("brick", dict(path=cs.PATH_BRICK)), ("brick_g1", dict(path=cs.PATH_BRICK, brick_groups=1)),
+            ("rows", dict(path=cs.PATH_ROWS)), ("auto", dict())]
+
+
+def test_device_is_gfx950(cs, torch_cuda):
+    info = cs.device_info()
+    assert info["arch"].startswith("gfx950") and info["wave_size"] == 64 and info["num_cus"] > 0
+
+
+@pytest.mark.parametrize("cfg,scale", [(1, 1.0), (2, 1 / 16.0), (3, 1 / 16.0), (4, 1 / 32.0), (5, 1 / 128.0)])
+def test_configs_against_oracle(cs, orc, torch_cuda, cfg, scale):
+    A = cs.gen_config(cfg, scale)
+    N = cs.CONFIGS[cfg]["N"]
+    B = cs.gen_dense(cs.SEED_BASE + 100 + cfg, A.K, N, 2)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch_cuda, h, B, **kw)
+        err = cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, out)
+        assert np.isfinite(out).all() and err <= BERR, (cfg, name, err)
+
+
+@pytest.mark.parametrize("N", [1, 3, 16, 20, 32, 48, 64, 100, 128, 130, 131, 192, 256, 320, 512, 1024])
+def test_every_width(cs, orc, torch_cuda, N):
+    rng = np.random.default_rng(N)
+    M, K = 160, 256
+    rp, cl, vl = random_csr(rng, M, K, density=0.08)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for name, kw in _paths(cs):
+        out, plan = _run(cs, torch_cuda, h, B, **kw)
+        err = cs.backward_error(rp, cl, vl, B, ref, out)
+        assert err <= BERR, (N, name, err, plan.info)
+
+
+def test_exact_cases(cs, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    K, N = 128, 64
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    # A = I  =>  C = B bit for bit
+    I = csr_from_dense(np.eye(K, dtype=np.float32))
+    h = cs.HRPB(K, K, *I)
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch, h, B, **kw)
+        assert (out == B).all(), name
+    # all-ones A and B  =>  row nonzero counts, exact in any summation order
+    rp, cl, vl = random_csr(rng, 96, K, density=0.3, values="ones")
+    h = cs.HRPB(96, K, rp, cl, vl)
+    ones = np.ones((K, N), np.float32)
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch, h, ones, **kw)
+        assert (out == np.diff(rp.astype(np.int64))[:, None]).all(), name
+    # one-hot B picks out a column of A (catches a transposed or permuted operand)
+    rp, cl, vl = random_csr(rng, 64, K, density=0.2, values="ints")
+    h = cs.HRPB(64, K, rp, cl, vl)
+    E = np.zeros((K, 16), np.float32)
+    picks = rng.choice(K, 16, replace=False)
+    E[picks, np.arange(16)] = 1
+    D = np.zeros((64, K), np.float32)
+    for r in range(64):
+        D[r, cl[rp[r]:rp[r + 1]]] = vl[rp[r]:rp[r + 1]]
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch, h, E, **kw)
+        assert (out == D[:, picks]).all(), name
+    # small integers: equal to the oracle's HRPB-stream SpMM and to CSR exactly
+
+
+def test_integer_inputs_equal_oracle_bit_for_bit(cs, orc, torch_cuda):
+    rng = np.random.default_rng(17)
+    M, K, N = 256, 320, 96
+    rp, cl, vl = random_csr(rng, M, K, density=0.05, values="ints")
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    assert (orc.spmm_hrpb(h.as_dict(), B) == ref).all()
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch_cuda, h, B, **kw)
+        assert (out == ref).all(), name
+
+
+def test_reference_regime_metric(cs, orc, torch_cuda):
+    """A = 1 everywhere it is non-zero, B uniform in [0,1): the reference's own check."""
+    import os
+    from test_oracle_pins import GOLD
+    r = cs.MTX_READER(os.path.join(GOLD, "G67.mtx"))
+    for N in (32, 128, 512):                     # run.cu:16
+        B = cs.gen_dense(5 + N, r.K, N, 0)
+        ref = orc.spmm_csr(r.rowPtr, r.cols, r.vals, B)
+        h = cs.HRPB(r.M, r.K, r.rowPtr, r.cols, r.vals)
+        for name, kw in _paths(cs):
+            out, _ = _run(cs, torch_cuda, h, B, **kw)
+            assert cs.check_gemm_correctness_coo(ref, out) <= 1e-5, (N, name)
+
+
+def test_edge_shapes(cs, orc, torch_cuda):
+    from test_oracle_pins import _edge_cases
+    rng = np.random.default_rng(0)
+    for name, (M, K, rp, cl, vl) in sorted(_edge_cases().items()):
+        B = rng.standard_normal((K, 64)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        h = cs.HRPB(M, K, rp, cl, vl)
+        for pname, kw in _paths(cs):
+            out, _ = _run(cs, torch_cuda, h, B, **kw)
+            assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (name, pname)
+            assert (out[np.diff(rp.astype(np.int64)) == 0] == 0).all()      # empty rows are written as zeros
+
+
+def test_split_panels_combine_through_atomics(cs, orc, torch_cuda):
+    """A few very long panels among short ones: the planner cuts them and the pieces add up."""
+    rng = np.random.default_rng(8)
+    M, K, N = 512, 4096, 128
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1500 if r in (5, 300) else 4)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK)
+    assert plan.info["numAtomicChunks"] > 0
+    assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
+    # forcing tiny chunks everywhere, and the reference's own partition arithmetic
+    for kw in (dict(max_chunk_blocks=1), dict(max_chunk_blocks=3), dict(slots=64), dict(slots=864)):
+        out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, **kw)
+        assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, kw
+    # a second launch on the same output buffer must not accumulate on top of the first
+    import torch
+    dB = torch.from_numpy(B).cuda()
+    dC = torch.zeros((M, N), device="cuda")
+    plan = cs.SPMM_TC(h, N, path=cs.PATH_BRICK, max_chunk_blocks=2)
+    plan.run(dB, dC)
+    plan.run(dB, dC)
+    torch.cuda.synchronize()
+    assert cs.backward_error(rp, cl, vl, B, ref, dC.cpu().numpy()) <= BERR
+
+
+def test_csr_comparison_kernels(cs, orc, torch_cuda):
+    torch = torch_cuda
+    A = cs.gen_config(2, 1 / 16.0)
+    for N in (32, 100, 128):
+        B = cs.gen_dense(3, A.K, N, 2)
+        ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+        h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+        dB = torch.from_numpy(B).cuda()
+        for alg in (0, 1, 2):
+            dC = torch.full((A.M, N), float("nan"), device="cuda")
+            cs.csr_spmm_dev(alg, h, dB, dC)
+            torch.cuda.synchronize()
+            assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, dC.cpu().numpy()) <= BERR, (N, alg)
+        hC = np.zeros((A.M, N), np.float32)
+        ms = cs.GPU_CSR_cuSPARSE_NEW(A.rowPtr, A.cols, A.vals, A.nnz, B, hC, A.M, A.K, N, 3)
+        assert ms > 0 and cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, hC) <= BERR
+
+
+def test_full_size_headline_config(cs, orc, torch_cuda):
+    """The benchmark workload itself (65536-row stencil, N=128): oracle comparison plus two
+    size-independent properties -- column sums (1^T C = (1^T A) B) and linearity in B."""
+    torch = torch_cuda
+    A = cs.gen_config(2)
+    N = 128
+    B = cs.gen_dense(cs.SEED_BASE + 102, A.K, N, 2)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+    out, plan = _run(cs, torch, h, B)
+    assert plan.info["numAtomicChunks"] == 0
+    assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, out) <= BERR
+    colsum = np.zeros(A.K, np.float64)
+    np.add.at(colsum, A.cols.astype(np.int64), A.vals.astype(np.float64))
+    expect = colsum @ B.astype(np.float64)
+    got = out.astype(np.float64).sum(0)
+    scale = np.abs(colsum) @ np.abs(B.astype(np.float64))
+    assert (np.abs(got - expect) <= 1e-5 * scale).all()
+    B2 = cs.gen_dense(99, A.K, N, 1)
+    out2, _ = _run(cs, torch, h, B2)
+    out3, _ = _run(cs, torch, h, (2.0 * B + B2).astype(np.float32))
+    # 2B is exact in fp32, so A(2B + B2) differs from 2AB + AB2 only by rounding of the sums
+    lin = np.abs(out3.astype(np.float64) - (2.0 * out + out2))
+    assert lin.max() <= 1e-4 * max(1.0, float(np.abs(out3).max()))
+
+
+def test_plan_rejects_bad_arguments(cs, torch_cuda):
+    import torch
+    rp, cl, vl = random_csr(np.random.default_rng(1), 32, 32, density=0.2)
+    h = cs.HRPB(32, 32, rp, cl, vl)
+    with pytest.raises(cs.CuteError) as e:
+        cs.SPMM_TC(h, 0)
+    assert e.value.status == -2
+    with pytest.raises(cs.CuteError):
+        cs.SPMM_TC(h, 32, path=7)
+    plan = cs.SPMM_TC(h, 32)
+    with pytest.raises(ValueError):
+        plan.run(torch.zeros((32, 16), device="cuda"), torch.zeros((32, 32), device="cuda"))
