@@ -1,0 +1,149 @@
+#!/usr/bin/env python3
+"""Benchmark of the brick-blocked SpMM hot path on one MI355X.
+
+A step is one SpMM (C = A.B) over the headline workload: the 65536-row 9-point-stencil
+matrix with a dense 65536 x 128 fp32 B, inputs resident in HBM before timing starts.
+Prints ONE JSON line: GFLOP/s = 2.nnz.N / t, the HBM roofline of the dominant kernel
+(algorithmic bytes / per-launch kernel time from HIP events on the launch stream) and
+the CPU oracle timed on the host cores as a reported baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu] [--detail FILE]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(M, K, N, nnz):
+    """CSR values + column indices + row pointers read once, B read once, C written once."""
+    return nnz * 8 + (M + 1) * 4 + K * N * 4 + M * N * 4
+
+
+def recorded_traffic(workload):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), if a
+    record for this workload has been committed under profiles/."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        rec = json.load(open(path)).get(workload)
+        return None if rec is None else float(rec["fetch_bytes"]) + float(rec["write_bytes"])
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def cpu_baseline(A, B, budget_s=10.0):
+    """The CPU oracle (row-parallel CSR restatement of inc.h:71-83) on the host cores:
+    repeated full passes over the same workload for about `budget_s` seconds."""
+    import oracle
+    out = np.empty((A.M, B.shape[1]), np.float32)
+    oracle.spmm_csr(A.rowPtr, A.cols, A.vals, B, out=out)           # warm-up pass
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end or len(times) < 3:
+        t0 = time.perf_counter()
+        oracle.spmm_csr(A.rowPtr, A.cols, A.vals, B, out=out)
+        times.append(time.perf_counter() - t0)
+        if len(times) >= 2000:
+            break
+    t = float(np.median(times))
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return dict(value=2.0 * A.nnz * B.shape[1] / t / 1e9, unit="GFLOP/s", cores=cores, kind="port",
+                sample="%d full passes of the same workload (median)" % len(times)), out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--detail", default=None, help="also time every path and the CSR kernels; write JSON here")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (got --gpus %d); nothing here shards across GPUs" % args.gpus)
+
+    import torch
+    import cutespmm_ae_amd as cs
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    cfg = cs.CONFIGS[args.config]
+    A = cs.gen_config(args.config)
+    N = cfg["N"]
+    B = cs.gen_dense(cs.SEED_BASE + 100 + args.config, A.K, N, 2)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    dB = torch.from_numpy(B).cuda()
+    dC = torch.empty((A.M, N), device="cuda")
+    plan = cs.SPMM_TC(h, N)
+    stream = torch.cuda.current_stream()
+
+    for _ in range(args.warmup):
+        plan.run(dB, dC)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run(dB, dC)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    flops = 2.0 * A.nnz * N
+    value = flops / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel: per-launch duration from HIP events on the launch stream
+    ms = plan.time(dB, dC, warmup=5, iters=max(20, min(args.steps, 200)), stream=stream)
+    kernel_ms = float(np.mean(ms))
+    abytes = algorithmic_bytes(A.M, A.K, N, A.nnz)
+    achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+                    traffic=recorded_traffic(cfg["name"]), kernel="hrpb_brick_f32" if plan.info["numChunks"] else "csr_rows",
+                    kernel_ms=kernel_ms, kernel_ms_median=float(np.median(ms)), algorithmic_bytes=abytes)
+
+    out = dict(metric="SpMM GFLOP/s (2*nnz*N/t) on 1 MI355X", value=value, unit="GFLOP/s", n_gpus=1,
+               steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
+               scaling="weak", vs_baseline=None, dtype="f32", data="synthetic (seeded generator)",
+               config=dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, blocks=h.numBlocks,
+                           bricks=h.num_bricks, plan={k: plan.info[k] for k in
+                                                      ("slabWidth", "numSlabs", "numChunks", "numAtomicChunks",
+                                                       "numBrickPanels", "numRowPanelsSparse")}),
+               roofline=roofline)
+
+    ref = None
+    if not args.no_cpu:
+        out["cpu_baseline"], ref = cpu_baseline(A, B)
+        got = dC.cpu().numpy()
+        out["backward_error_vs_oracle"] = cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, got)
+        out["reference_metric_vs_oracle"] = cs.check_gemm_correctness_coo(ref, got)
+
+    if args.detail:
+        detail = dict(workload=cfg["name"], paths={}, csr={})
+        for name, kw in (("brick_groups2", dict(path=cs.PATH_BRICK, brick_groups=2)),
+                         ("brick_groups1", dict(path=cs.PATH_BRICK, brick_groups=1)),
+                         ("rows", dict(path=cs.PATH_ROWS)), ("auto", dict())):
+            p = cs.SPMM_TC(h, N, **kw)
+            t = p.time(dB, dC, warmup=5, iters=50, stream=stream)
+            detail["paths"][name] = dict(median_us=float(np.median(t)) * 1e3, mean_us=float(np.mean(t)) * 1e3,
+                                         gflops=flops / (float(np.median(t)) * 1e-3) / 1e9, info=p.info)
+        for alg, name in ((0, "thread_per_element"), (1, "wave_per_row_scalar"), (2, "wave_per_row_vector")):
+            t = cs.csr_spmm_time(alg, h, dB, dC, warmup=3, iters=30, stream=stream)
+            detail["csr"][name] = dict(median_us=float(np.median(t)) * 1e3,
+                                       gflops=flops / (float(np.median(t)) * 1e-3) / 1e9)
+        best = max(v["gflops"] for v in detail["csr"].values())
+        detail["best_simple_csr_gflops"] = best
+        detail["speedup_over_best_simple_csr"] = detail["paths"]["auto"]["gflops"] / best
+        with open(args.detail, "w") as f:
+            json.dump(detail, f, indent=1)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -87,6 +87,7 @@ struct cute_spmm_plan {
     const cute_hrpb_dev *d = nullptr;
     cute_plan_info info{};
     int vec = 4, ng = 1;                // brick kernel shape
+    int pipeline = 2;                   // 1: resident variant, 2: pipelined variant
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
@@ -222,8 +223,11 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->d = d;
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
-    p->ng = (p->vec == 4 && N >= 128) ? 2 : 1;
+    p->ng = 1;   // one 16-lane column group per lane measured faster than two on every benchmark matrix
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
+    if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
+    p->pipeline = t.pipeline ? int(t.pipeline) : 2;
+    if (p->pipeline == 1) p->ng = 1;   // the resident variant's register budget holds one column group
     const uint32_t slab = 16u * p->vec * p->ng;
     const uint32_t num_slabs = (N + slab - 1) / slab;
     // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
@@ -338,9 +342,14 @@ void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipS
     const uint64_t items = uint64_t(p->info.numChunks) * p->info.numSlabs;
     const uint32_t groups = uint32_t((items + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup);
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
-    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
-                       dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
-                       p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+    if (p->pipeline == 1 && NG == 1)
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_resident<VEC, 1, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
+                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
+                           p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+    else
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
+                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
+                           p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
 }
 
 template <int VEC, int NG>
@@ -350,7 +359,7 @@ void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream
     else launch_brick_full<VEC, NG, false>(p, dB, dC, s);
 }
 
-template <int VEC>
+template <int VEC, bool BATCHED>
 void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
                      const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
 {
@@ -358,8 +367,12 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
     const dim3 grid(uint32_t((lanes + 255) / 256)), block(256);
 #define CUTE_ROWS_CASE(LL)                                                                                        \
     case LL:                                                                                                      \
-        hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, row_list, num_rows, slabs, rp, cl, vl, \
-                           dB, dC, N);                                                                            \
+        if (BATCHED)                                                                                              \
+            hipLaunchKernelGGL((cute_dev::csr_rows_batched<VEC, LL, 8>), grid, block, 0, s, row_list, num_rows,    \
+                               slabs, rp, cl, vl, dB, dC, N);                                                     \
+        else                                                                                                      \
+            hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, row_list, num_rows, slabs, rp,    \
+                               cl, vl, dB, dC, N);                                                                \
         break;
     switch (logl) {
         CUTE_ROWS_CASE(0) CUTE_ROWS_CASE(1) CUTE_ROWS_CASE(2) CUTE_ROWS_CASE(3)
@@ -368,12 +381,14 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
 #undef CUTE_ROWS_CASE
 }
 
+// batched: the library's sparse-panel kernel; otherwise the plain comparison kernel
+template <bool BATCHED>
 void launch_rows(int vec, int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
                  const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
 {
-    if (vec == 4) launch_rows_vec<4>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
-    else if (vec == 2) launch_rows_vec<2>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
-    else launch_rows_vec<1>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    if (vec == 4) launch_rows_vec<4, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    else if (vec == 2) launch_rows_vec<2, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    else launch_rows_vec<1, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
 }
 
 int check_launch(const char *what)
@@ -401,7 +416,7 @@ int csr_launch(int alg, const uint32_t *rp, const uint32_t *cl, const float *vl,
             uint32_t need = (N + vec - 1) / vec, logl = 0;
             while ((1u << logl) < need && logl < 6) ++logl;
             const uint32_t w = (1u << logl) * vec;
-            launch_rows(vec, int(logl), nullptr, M, (N + w - 1) / w, rp, cl, vl, dB, dC, N, s);
+            launch_rows<false>(vec, int(logl), nullptr, M, (N + w - 1) / w, rp, cl, vl, dB, dC, N, s);
             break;
         }
         default: return CUTE_ERR_ARG;
@@ -454,7 +469,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         else launch_brick<1, 1>(p, dB, dC, s);
     }
     if (p->numRows) {
-        launch_rows(p->rows_vec, p->rows_logl, p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
+        launch_rows<true>(p->rows_vec, p->rows_logl, p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
                     p->d->dCsrVals, dB, dC, N, s);
     }
     return check_launch("spmm launch");

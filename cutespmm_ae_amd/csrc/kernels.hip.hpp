@@ -111,26 +111,71 @@ __device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x
 // MFMA tile v of that group therefore holds the columns {.. + j*VEC + v}, and after the
 // MFMA lane L holds rows 4g..4g+3 of exactly those VEC columns -> one vector store per row.
 // FULL: N is a multiple of the slab width, so no column guard is compiled in.
+struct BrickItem {
+    uint32_t start, end, panel, atomic, col0;
+    bool valid;
+};
+
+template <int VEC, int NG>
+__device__ __forceinline__ BrickItem brick_item(const uint4 *__restrict__ chunks, uint32_t num_chunks,
+                                                uint32_t num_slabs, uint32_t groups_per_xcd, uint32_t lane)
+{
+    BrickItem it;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const uint32_t group = xcd_contiguous_id(blockIdx.x, groups_per_xcd);
+    const uint64_t item = uint64_t(group) * kWavesPerGroup + wave;
+    it.valid = item < uint64_t(num_chunks) * num_slabs;
+    if (!it.valid) return it;
+    const uint32_t chunk = uint32_t(item / num_slabs);
+    const uint32_t slab = uint32_t(item % num_slabs);
+    const uint4 ck = chunks[chunk];
+    it.start = __builtin_amdgcn_readfirstlane(ck.x);
+    it.end = __builtin_amdgcn_readfirstlane(ck.y);
+    it.panel = __builtin_amdgcn_readfirstlane(ck.z);
+    it.atomic = __builtin_amdgcn_readfirstlane(ck.w);
+    it.col0 = slab * (16u * VEC * NG) + (lane & 15u) * VEC;
+    return it;
+}
+
+template <int VEC, int NG, bool FULL>
+__device__ __forceinline__ void brick_store(const BrickItem &it, const f32x4 (&acc)[NG][VEC], float *__restrict__ C,
+                                            uint32_t N, uint32_t lane)
+{
+    typedef typename Vec<VEC>::type V;
+    const uint32_t row0 = it.panel * 16u + (lane >> 4) * 4u;
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng) {
+        const uint32_t c = it.col0 + uint32_t(ng) * 16u * VEC;
+        if (!FULL && c >= N) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float *dst = C + size_t(row0 + r) * N + c;
+            if (it.atomic) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
+            } else {
+                V out;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
+                *reinterpret_cast<V *>(dst) = out;
+            }
+        }
+    }
+}
+
+// Variant "pipelined": two operand sets per wavefront ping-pong, so a wavefront overlaps its
+// own loads with its own MFMAs.  Best when work items are long (many blocks per chunk) and
+// few wavefronts fit per SIMD anyway.
 template <int VEC, int NG, bool FULL>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
     const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
     float *__restrict__ C, uint32_t N)
 {
-    typedef typename Vec<VEC>::type V;
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t group = xcd_contiguous_id(blockIdx.x, groups_per_xcd);
-    const uint64_t item = uint64_t(group) * kWavesPerGroup + wave;
-    if (item >= uint64_t(num_chunks) * num_slabs) return;
-    const uint32_t chunk = uint32_t(item / num_slabs);
-    const uint32_t slab = uint32_t(item % num_slabs);
-    const uint4 ck = chunks[chunk];
-    const uint32_t start = __builtin_amdgcn_readfirstlane(ck.x);
-    const uint32_t end = __builtin_amdgcn_readfirstlane(ck.y);
-    const uint32_t panel = __builtin_amdgcn_readfirstlane(ck.z);
-    const uint32_t atomic = __builtin_amdgcn_readfirstlane(ck.w);
-    const uint32_t col0 = slab * (16u * VEC * NG) + (lane & 15u) * VEC;
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, num_slabs, groups_per_xcd, lane);
+    if (!it.valid) return;
+    const uint32_t end = it.end, col0 = it.col0;
 
     f32x4 acc[NG][VEC];
 #pragma unroll
@@ -144,7 +189,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     // scheduling barriers really keep each load group ahead of the MFMAs that hide it.
     BlockOperands<VEC, NG> opA, opB;
     BlockHeader hd, hn;
-    uint32_t blk = start;
+    uint32_t blk = it.start;
     if (blk < end) {
         hd = load_header(hdr, blk, lane);
         if (blk + 1 < end) hn = load_header(hdr, blk + 1, lane);
@@ -190,26 +235,44 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
         __builtin_amdgcn_sched_barrier(0);
         mfma_block<VEC, NG>(opA, acc, lane);
     }
+    brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
+}
 
-    const uint32_t row0 = panel * 16u + (lane >> 4) * 4u;
+// Variant "resident": one operand set per wavefront and a register budget that lets eight
+// wavefronts share a SIMD, so that for short work items (a handful of blocks per panel) every
+// item of the launch is resident at once and the SIMD hides one wavefront's loads behind the
+// others' MFMAs.  Header lines still run two blocks ahead.
+template <int VEC, int NG, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_resident(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
+    const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
+    float *__restrict__ C, uint32_t N)
+{
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, num_slabs, groups_per_xcd, lane);
+    if (!it.valid) return;
+    const uint32_t end = it.end, col0 = it.col0;
+
+    f32x4 acc[NG][VEC];
 #pragma unroll
-    for (int ng = 0; ng < NG; ++ng) {
-        const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
-        if (!FULL && c >= N) continue;
+    for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float *dst = C + size_t(row0 + r) * N + c;
-            if (atomic) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
-            } else {
-                V out;
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
-                *reinterpret_cast<V *>(dst) = out;
-            }
-        }
+        for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
+
+    BlockOperands<VEC, NG> op;
+    BlockHeader hd, hn;
+    uint32_t blk = it.start;
+    if (blk < end) {
+        hd = load_header(hdr, blk, lane);
+        hn = load_header(hdr, min(blk + 1, end - 1), lane);
     }
+    for (; blk < end; ++blk) {
+        load_operands<VEC, NG, FULL>(op, hd, vals, B, N, col0, lane);
+        hd = hn;
+        hn = load_header(hdr, min(blk + 2, end - 1), lane);   // clamped: the loop stays branch-free
+        mfma_block<VEC, NG>(op, acc, lane);
+    }
+    brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
 }
 
 // Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).
@@ -257,6 +320,55 @@ __global__ __launch_bounds__(256) void csr_rows(const uint32_t *__restrict__ row
                 const V b = *reinterpret_cast<const V *>(B + size_t(c) * N + c0);
                 acc += a * b;
             }
+        }
+    }
+    if (live) *reinterpret_cast<V *>(C + size_t(row) * N + c0) = acc;
+}
+
+// The sparse-panel kernel of the library: same work split as csr_rows, but the nonzeros of a
+// row are consumed in batches whose B-row loads are all issued before the first FMA, so a
+// row costs about one memory round trip per batch instead of one per nonzero.  Each C
+// element still accumulates its row in storage order.
+template <int VEC, int LOG_L, int BATCH>
+__global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restrict__ row_list, uint32_t num_rows,
+                                                        uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+                                                        const uint32_t *__restrict__ cols,
+                                                        const float *__restrict__ vals, const float *__restrict__ B,
+                                                        float *__restrict__ C, uint32_t N)
+{
+    typedef typename Vec<VEC>::type V;
+    constexpr uint32_t L = 1u << LOG_L;
+    constexpr uint32_t STEP = BATCH < int(L) ? uint32_t(BATCH) : L;
+    const uint32_t t = threadIdx.x & (L - 1);
+    const uint64_t gid = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> LOG_L;
+    if (gid >= uint64_t(num_rows) * num_slabs) return;
+    const uint32_t ridx = uint32_t(gid / num_slabs);
+    const uint32_t slab = uint32_t(gid % num_slabs);
+    const uint32_t row = row_list ? row_list[ridx] : ridx;
+    const uint32_t c0 = slab * L * VEC + t * VEC;
+    const bool live = c0 < N;
+    const uint32_t s = rowPtr[row], e = rowPtr[row + 1];
+    const float *bcol = B + c0;
+    V acc = V(0.0f);
+    for (uint32_t base = s; base < e; base += L) {
+        const uint32_t mine = base + t;
+        uint32_t my_col = 0;
+        float my_val = 0.0f;
+        if (mine < e) { my_col = cols[mine]; my_val = vals[mine]; }
+        const uint32_t cnt = min(L, e - base);
+        for (uint32_t q0 = 0; q0 < cnt; q0 += STEP) {
+            V b[STEP];
+            float a[STEP];
+#pragma unroll
+            for (uint32_t u = 0; u < STEP; ++u) {
+                // lanes past the end of the row hold (col 0, val 0): their slot is skipped
+                const uint32_t c = __shfl(my_col, int(q0 + u), int(L));
+                a[u] = __shfl(my_val, int(q0 + u), int(L));
+                b[u] = V(0.0f);
+                if (live && q0 + u < cnt) b[u] = *reinterpret_cast<const V *>(bcol + size_t(c) * N);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < STEP; ++u) acc += a[u] * b[u];
         }
     }
     if (live) *reinterpret_cast<V *>(C + size_t(row) * N + c0) = acc;

@@ -187,7 +187,8 @@ typedef struct cute_tunables {
     uint32_t slots;            /* resident work items assumed by the partition; 0: derive from device */
     uint32_t max_chunk_blocks; /* upper bound on blocks per work item; 0: none            */
     uint32_t brick_groups;     /* 16-lane column groups per lane in the brick kernel (1 or 2); 0: default */
-    uint32_t reserved[2];
+    uint32_t pipeline;         /* brick kernel variant: 1 resident (one operand set, 8 wavefronts/SIMD), 2 pipelined; 0: default */
+    uint32_t reserved[1];
 } cute_tunables;
 
 typedef struct cute_plan_info {
