@@ -31,7 +31,7 @@ def algorithmic_bytes(M, K, N, nnz):
 def recorded_traffic(workload):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), if a
     record for this workload has been committed under profiles/."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_%s.json" % workload)
     try:
         rec = json.load(open(path)).get(workload)
         return None if rec is None else float(rec["fetch_bytes"]) + float(rec["write_bytes"])

@@ -47,8 +47,10 @@ def build_driver():
     src = os.path.join(CSRC, "run_cute.cpp")
     if not os.path.exists(src):
         return None
-    _run([HIPCC, "-x", "c++", src] + COMMON + ["-I", os.path.join(ROOT, "include"), "-o", DRIVER,
-                                                "-L", HERE, "-lcutespmm", "-Wl,-rpath,$ORIGIN"])
+    rocm = os.path.dirname(os.path.dirname(os.path.realpath(HIPCC)))
+    _run([HIPCC, "-x", "c++", src, "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include")] + COMMON +
+         ["-I", os.path.join(ROOT, "include"), "-o", DRIVER, "-L", HERE, "-lcutespmm",
+          "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN"])
     return DRIVER
 
 
