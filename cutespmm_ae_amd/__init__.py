@@ -27,6 +27,10 @@ ABI_SYMBOLS = [
     "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run",
     "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
     "cute_device_info",
+    "cute_coo_read", "cute_coo_save_mtx", "cute_coo_release", "cute_coo_to_csr", "cute_csr_i32_release",
+    "cute_csr_to_dense", "cute_csr_count_blocks", "cute_csr_to_bcsr", "cute_bcsr_release",
+    "cute_blocked_ell_build", "cute_blocked_ell_to_dense", "cute_blocked_ell_release",
+    "cute_splitter_split", "cute_split_release", "cute_classify_blocks", "cute_sequential_spmm",
 ]
 
 u32p = C.POINTER(C.c_uint32)
@@ -70,6 +74,39 @@ class cute_plan_info(C.Structure):
                 ("numAtomicChunks", C.c_uint32), ("numBrickPanels", C.c_uint32), ("numRowPanelsSparse", C.c_uint32),
                 ("numEmptyPanels", C.c_uint32), ("slots", C.c_uint32), ("precision", C.c_uint32),
                 ("path", C.c_uint32), ("reserved", C.c_uint32 * 5)]
+
+
+i32p = C.POINTER(C.c_int32)
+
+
+class cute_coo(C.Structure):
+    _fields_ = [("dimY", C.c_int32), ("dimX", C.c_int32), ("nnz", C.c_int32), ("rows", i32p), ("cols", i32p),
+                ("values", f32p)]
+
+
+class cute_csr_i32(C.Structure):
+    _fields_ = [("nrows", C.c_int32), ("ncols", C.c_int32), ("nnz", C.c_int32), ("rowPtr", i32p), ("cols", i32p),
+                ("values", f32p)]
+
+
+class cute_bcsr(C.Structure):
+    _fields_ = [("R", C.c_int32), ("C", C.c_int32), ("nrows", C.c_int32), ("ncols", C.c_int32), ("nblks", C.c_int32),
+                ("rowPtr", i32p), ("cols", i32p), ("values", f32p)]
+
+
+class cute_blocked_ell(C.Structure):
+    _fields_ = [("blockSize", C.c_int32), ("height", C.c_int32), ("width", C.c_int32), ("numBlocks", C.c_int32),
+                ("numElems", C.c_int32), ("ellColIdx", i32p), ("ellValues", f32p)]
+
+
+class cute_split(C.Structure):
+    _fields_ = [("totalTiles", C.c_int32), ("numHeavyTiles", C.c_int32), ("numHeavyElems", C.c_int32),
+                ("numLightTiles", C.c_int32), ("numLightElems", C.c_int32), ("heavy", cute_coo), ("light", cute_coo)]
+
+
+class cute_block_class(C.Structure):
+    _fields_ = [("blockRow", C.c_int32), ("blockCol", C.c_int32), ("nnz", C.c_int32), ("underloads", C.c_int32),
+                ("overloads", C.c_int32), ("kind", C.c_int32)]
 
 
 PATH_AUTO, PATH_BRICK, PATH_ROWS = 0, 1, 2
@@ -131,6 +168,26 @@ def load_library():
     lib.cute_csr_spmm_time.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p,
                                        C.c_int, C.c_int, f32p]
     lib.cute_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_size_t]
+    lib.cute_coo_read.argtypes = [C.c_char_p, C.POINTER(cute_coo)]
+    lib.cute_coo_save_mtx.argtypes = [C.POINTER(cute_coo), C.c_char_p]
+    lib.cute_coo_release.argtypes = [C.POINTER(cute_coo)]
+    lib.cute_coo_to_csr.argtypes = [C.POINTER(cute_coo), C.POINTER(cute_csr_i32)]
+    lib.cute_csr_i32_release.argtypes = [C.POINTER(cute_csr_i32)]
+    lib.cute_csr_to_dense.argtypes = [C.POINTER(cute_csr_i32), f32p]
+    lib.cute_csr_count_blocks.restype = C.c_int64
+    lib.cute_csr_count_blocks.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32]
+    lib.cute_csr_to_bcsr.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32, C.POINTER(cute_bcsr)]
+    lib.cute_bcsr_release.argtypes = [C.POINTER(cute_bcsr)]
+    lib.cute_blocked_ell_build.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.POINTER(cute_blocked_ell)]
+    lib.cute_blocked_ell_to_dense.argtypes = [C.POINTER(cute_blocked_ell), C.c_int32, f32p]
+    lib.cute_blocked_ell_release.argtypes = [C.POINTER(cute_blocked_ell)]
+    lib.cute_splitter_split.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32, C.POINTER(cute_split)]
+    lib.cute_split_release.argtypes = [C.POINTER(cute_split)]
+    lib.cute_classify_blocks.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_float, C.c_float,
+                                         C.POINTER(C.POINTER(cute_block_class)), C.POINTER(C.c_int64)]
+    lib.cute_sequential_spmm.restype = C.c_float
+    lib.cute_sequential_spmm.argtypes = [C.POINTER(cute_csr_i32), C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                         C.POINTER(C.c_double), C.c_int32, C.c_int32, C.c_int32]
     _lib = lib
     return lib
 
@@ -483,3 +540,160 @@ def device_info():
     name = C.create_string_buffer(64)
     _check(load_library().cute_device_info(C.byref(cus), C.byref(ws), name, 64), "cute_device_info")
     return dict(num_cus=cus.value, wave_size=ws.value, arch=name.value.decode())
+
+
+# --------------------------------------------------------------------------------------
+# second API family (inc/SparseCoo.hpp, inc/CSR.hpp, inc/prepareBlkEll.hpp, inc/splitter.hpp)
+# Arrays are copied into numpy-owned memory; the library's copies are released at once.
+# --------------------------------------------------------------------------------------
+def _take(ptr, n, dtype):
+    n = int(n)
+    return np.ctypeslib.as_array(ptr, shape=(n,)).astype(dtype, copy=True) if n else np.zeros(0, dtype)
+
+
+def _coo_fields(raw):
+    return (raw.dimY, raw.dimX, raw.nnz, _take(raw.rows, raw.nnz, np.int32), _take(raw.cols, raw.nnz, np.int32),
+            _take(raw.values, raw.nnz, np.float32))
+
+
+class SparseCoo:
+    """``SparseCoo(path)`` (inc/SparseCoo.hpp:91-157) or ``SparseCoo(dimY, dimX, rows, cols, values)``."""
+
+    def __init__(self, *args):
+        if len(args) == 1:
+            raw = cute_coo()
+            _check(load_library().cute_coo_read(os.fsencode(args[0]), C.byref(raw)), "cute_coo_read(%s)" % args[0])
+            self.dimY, self.dimX, self.nnz, self.rows, self.cols, self.values = _coo_fields(raw)
+            load_library().cute_coo_release(C.byref(raw))
+        else:
+            self.dimY, self.dimX = int(args[0]), int(args[1])
+            self.rows, self.cols, self.values = _as(args[2], np.int32), _as(args[3], np.int32), _as(args[4], np.float32)
+            self.nnz = len(self.rows)
+
+    def _raw(self):
+        return cute_coo(self.dimY, self.dimX, self.nnz, _ptr(self.rows, i32p), _ptr(self.cols, i32p),
+                        _ptr(self.values, f32p))
+
+    def save_mtx(self, path):
+        raw = self._raw()
+        _check(load_library().cute_coo_save_mtx(C.byref(raw), os.fsencode(path)), "cute_coo_save_mtx")
+
+
+class CSR_Matrix:
+    """``CSR_Matrix(coo)`` = coo2CSR (inc/CSR.hpp:162-187); fields nrows, ncols, nnz, rowPtr, cols, values."""
+
+    def __init__(self, coo=None, nrows=None, ncols=None, rowPtr=None, cols=None, values=None):
+        if coo is not None:
+            raw, src = cute_csr_i32(), coo._raw()
+            _check(load_library().cute_coo_to_csr(C.byref(src), C.byref(raw)), "cute_coo_to_csr")
+            self.nrows, self.ncols, self.nnz = raw.nrows, raw.ncols, raw.nnz
+            self.rowPtr = _take(raw.rowPtr, raw.nrows + 1, np.int32)
+            self.cols, self.values = _take(raw.cols, raw.nnz, np.int32), _take(raw.values, raw.nnz, np.float32)
+            load_library().cute_csr_i32_release(C.byref(raw))
+        else:
+            self.nrows, self.ncols = int(nrows), int(ncols)
+            self.rowPtr, self.cols, self.values = _as(rowPtr, np.int32), _as(cols, np.int32), _as(values, np.float32)
+            self.nnz = len(self.cols)
+
+    def _raw(self):
+        return cute_csr_i32(self.nrows, self.ncols, self.nnz, _ptr(self.rowPtr, i32p), _ptr(self.cols, i32p),
+                            _ptr(self.values, f32p))
+
+    def ToDense(self):
+        dense = np.zeros((self.nrows, self.ncols), np.float32)
+        raw = self._raw()
+        _check(load_library().cute_csr_to_dense(C.byref(raw), _ptr(dense, f32p)), "cute_csr_to_dense")
+        return dense
+
+    def csr_count_blocks(self, R, Cc):
+        raw = self._raw()
+        n = load_library().cute_csr_count_blocks(C.byref(raw), int(R), int(Cc))
+        if n < 0:
+            raise CuteError(int(n), "cute_csr_count_blocks")
+        return int(n)
+
+    def to_BCSR(self, R, Cc):
+        raw, out = self._raw(), cute_bcsr()
+        _check(load_library().cute_csr_to_bcsr(C.byref(raw), int(R), int(Cc), C.byref(out)), "cute_csr_to_bcsr")
+        res = dict(R=out.R, C=out.C, BCSR_nrows=out.nrows, BCSR_ncols=out.ncols, BCSR_nblks=out.nblks,
+                   BCSR_rowPtr=_take(out.rowPtr, out.nrows + 1, np.int32), BCSR_cols=_take(out.cols, out.nblks, np.int32),
+                   BCSR_values=_take(out.values, out.nblks * out.R * out.C, np.float32))
+        load_library().cute_bcsr_release(C.byref(out))
+        return res
+
+    def sequentioal_spmm(self, B):
+        """inc/SPMM.cuh:123-187: double-precision CPU product; returns (C, ms)."""
+        B = _as(B, np.float64)
+        vals = _as(self.values, np.float64)
+        Cm = np.zeros((self.nrows, B.shape[1]), np.float64)
+        raw = self._raw()
+        dp = C.POINTER(C.c_double)
+        ms = load_library().cute_sequential_spmm(C.byref(raw), _ptr(vals, dp), _ptr(B, dp), _ptr(Cm, dp), self.nrows,
+                                                 self.ncols, B.shape[1])
+        if ms < 0:
+            raise CuteError(int(ms), "cute_sequential_spmm")
+        return Cm, ms
+
+
+class preprocess:
+    """``preprocess(csr, BlockSize)``: Blocked-ELL (inc/prepareBlkEll.hpp:185-196) with the getters of :267-290."""
+
+    def __init__(self, A_CSR, BlockSize):
+        raw, out = A_CSR._raw(), cute_blocked_ell()
+        _check(load_library().cute_blocked_ell_build(C.byref(raw), int(BlockSize), C.byref(out)), "cute_blocked_ell_build")
+        self.BlockSize, self._h, self._w = out.blockSize, out.height, out.width
+        self._nb, self._ne, self._ncols = out.numBlocks, out.numElems, A_CSR.ncols
+        self._idx = _take(out.ellColIdx, out.height * out.width, np.int32).reshape(out.height, out.width)
+        self._val = _take(out.ellValues, out.height * out.blockSize * out.width * out.blockSize,
+                          np.float32).reshape(out.height * out.blockSize, out.width * out.blockSize)
+        load_library().cute_blocked_ell_release(C.byref(out))
+
+    def get_ellColIdx(self): return self._idx
+    def get_ellColIdx_height(self): return self._h
+    def get_ellColIdx_width(self): return self._w
+    def get_ellValues(self): return self._val
+    def get_num_blocks(self): return self._nb
+    def get_num_elems(self): return self._ne
+
+    def blockedELLToDense(self):
+        dense = np.zeros((self._h * self.BlockSize, self._ncols), np.float32)
+        raw = cute_blocked_ell(self.BlockSize, self._h, self._w, self._nb, self._ne, _ptr(self._idx, i32p),
+                               _ptr(self._val, f32p))
+        _check(load_library().cute_blocked_ell_to_dense(C.byref(raw), self._ncols, _ptr(dense, f32p)),
+               "cute_blocked_ell_to_dense")
+        return dense
+
+
+class Splitter:
+    """``Splitter(csr, tile_size, NNZThreshold)`` (inc/splitter.hpp:126-142) with its seven getters."""
+
+    def __init__(self, A_CSR, tile_size, NNZThreshold):
+        raw, out = A_CSR._raw(), cute_split()
+        _check(load_library().cute_splitter_split(C.byref(raw), int(tile_size), int(NNZThreshold), C.byref(out)),
+               "cute_splitter_split")
+        self._c = (out.totalTiles, out.numHeavyTiles, out.numHeavyElems, out.numLightTiles, out.numLightElems)
+        self._heavy = SparseCoo(*_coo_fields(out.heavy)[:2], *_coo_fields(out.heavy)[3:])
+        self._light = SparseCoo(*_coo_fields(out.light)[:2], *_coo_fields(out.light)[3:])
+        load_library().cute_split_release(C.byref(out))
+
+    def get_total_tiles(self): return self._c[0]
+    def get_num_heavy_tiles(self): return self._c[1]
+    def get_num_heavy_elems(self): return self._c[2]
+    def get_num_light_tiles(self): return self._c[3]
+    def get_num_light_elems(self): return self._c[4]
+    def get_heavyMatrix(self): return self._heavy
+    def get_lightMatrix(self): return self._light
+
+
+def classify_blocks(A_CSR, BlockSize, deviation_threshold, underload_dominance):
+    """inc/preprocess.hpp:64-193 -> int32 array [n, 6]: blockRow, blockCol, nnz, underloads, overloads, kind."""
+    raw = A_CSR._raw()
+    out, n = C.POINTER(cute_block_class)(), C.c_int64()
+    _check(load_library().cute_classify_blocks(C.byref(raw), int(BlockSize), float(deviation_threshold),
+                                               float(underload_dominance), C.byref(out), C.byref(n)),
+           "cute_classify_blocks")
+    arr = np.zeros((n.value, 6), np.int32)
+    if n.value:
+        arr[:] = np.ctypeslib.as_array(C.cast(out, i32p), shape=(n.value, 6))
+    load_library().cute_free(C.cast(out, C.c_void_p))
+    return arr

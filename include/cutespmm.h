@@ -156,6 +156,75 @@ int cute_gen_matrix(int kind, uint64_t seed, uint32_t p0, uint32_t p1, uint32_t 
 int cute_gen_dense(uint64_t seed, int dist, uint64_t count, float *out);
 
 /* ------------------------------------------------------------------------------------
+ * host: the reference's second API family (signed int indices, dimensions as in the file,
+ * values kept).  fp32 instantiation of the templates.
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_coo {          /* SparseCoo<float>, inc/SparseCoo.hpp:41-388 (SoA form, :250-261) */
+    int32_t dimY, dimX, nnz;       /* rows, columns, entries (header count + mirrored entries)         */
+    int32_t *rows, *cols;
+    float *values;
+} cute_coo;
+
+typedef struct cute_csr_i32 {      /* CSR_Matrix<float>, inc/CSR.hpp:42-51                              */
+    int32_t nrows, ncols, nnz;
+    int32_t *rowPtr, *cols;
+    float *values;
+} cute_csr_i32;
+
+/* SparseCoo<T>(path), inc/SparseCoo.hpp:91-157: keeps values (1.0 if absent), mirrors
+ * symmetric files, sorts by (row, col). */
+int cute_coo_read(const char *path, cute_coo *out);
+/* save_mtx, inc/SparseCoo.hpp:263-285 ("real general", 1-based, one entry per line). */
+int cute_coo_save_mtx(const cute_coo *coo, const char *path);
+void cute_coo_release(cute_coo *coo);
+/* CSR_Matrix<T>::coo2CSR, inc/CSR.hpp:162-187 (sorts a copy by (row, col) first). */
+int cute_coo_to_csr(const cute_coo *coo, cute_csr_i32 *out);
+void cute_csr_i32_release(cute_csr_i32 *csr);
+/* ToDense, inc/CSR.hpp:315-329: dense[nrows*ncols] row-major, caller-zeroed. */
+int cute_csr_to_dense(const cute_csr_i32 *csr, float *dense);
+/* csr_count_blocks, inc/CSR.hpp:728-743: number of non-empty R x C blocks (< 0: status). */
+int64_t cute_csr_count_blocks(const cute_csr_i32 *csr, int32_t R, int32_t C);
+
+typedef struct cute_bcsr {         /* to_BCSR outputs, inc/CSR.hpp:760-810                               */
+    int32_t R, C, nrows, ncols, nblks;      /* block shape, block rows, block columns, blocks         */
+    int32_t *rowPtr, *cols;                 /* [nrows+1], [nblks]                                      */
+    float *values;                          /* [nblks*R*C], each block row-major                       */
+} cute_bcsr;
+int cute_csr_to_bcsr(const cute_csr_i32 *csr, int32_t R, int32_t C, cute_bcsr *out);
+void cute_bcsr_release(cute_bcsr *b);
+
+typedef struct cute_blocked_ell {  /* preprocess<float>, inc/prepareBlkEll.hpp:15-291                    */
+    int32_t blockSize, height, width;       /* ellColIdx is [height x width]                           */
+    int32_t numBlocks, numElems;
+    int32_t *ellColIdx;                     /* ascending block columns per block row, -1 padded        */
+    float *ellValues;                       /* [height*blockSize x width*blockSize] row-major          */
+} cute_blocked_ell;
+int cute_blocked_ell_build(const cute_csr_i32 *csr, int32_t blockSize, cute_blocked_ell *out);
+/* blockedELLToDense, inc/prepareBlkEll.hpp:242-266: dense[height*blockSize x ncols], caller-zeroed. */
+int cute_blocked_ell_to_dense(const cute_blocked_ell *e, int32_t ncols, float *dense);
+void cute_blocked_ell_release(cute_blocked_ell *e);
+
+typedef struct cute_split {        /* Splitter, inc/splitter.hpp:14-187                                  */
+    int32_t totalTiles, numHeavyTiles, numHeavyElems, numLightTiles, numLightElems;
+    cute_coo heavy, light;                  /* tile nnz >= threshold / < threshold; CSR order kept     */
+} cute_split;
+int cute_splitter_split(const cute_csr_i32 *csr, int32_t tile_size, int32_t nnz_threshold, cute_split *out);
+void cute_split_release(cute_split *s);
+
+typedef struct cute_block_class {  /* one non-empty blockSize^2 block, inc/preprocess.hpp:64-193          */
+    int32_t blockRow, blockCol, nnz, underloads, overloads;
+    int32_t kind;                           /* 0 dense, 1 2:4-sparse, 2 very sparse                    */
+} cute_block_class;
+/* Band statistics (:64-151) and the classification rule (:172-193); blocks sorted by
+ * (blockRow, blockCol).  *out is an array of *count entries, released with cute_free. */
+int cute_classify_blocks(const cute_csr_i32 *csr, int32_t blockSize, float deviation_threshold,
+                         float underload_dominance, cute_block_class **out, int64_t *count);
+
+/* sequentioal_spmm, inc/SPMM.cuh:123-187: double-precision CPU CSR SpMM; returns ms. */
+float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, const double *B, double *C,
+                           int32_t m, int32_t k, int32_t n);
+
+/* ------------------------------------------------------------------------------------
  * device: upload.        Replaces the cudaMalloc/cudaMemcpy tail of DATASTRUCT
  * (data.cu:327-334) and HRPB::freeDevice (data.cu:336-339).  Uploads the MFMA-tiled
  * layout, the per-panel descriptors and the borrowed CSR (for the sparse-panel path).

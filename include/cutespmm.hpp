@@ -134,3 +134,153 @@ inline float GPU_CSR_cuSPARSE_NEW(unsigned int *hA_csrOffsets, unsigned int *hA_
     if (ms < 0) throw cute::Error(int(ms), "GPU_CSR_cuSPARSE_NEW");
     return ms;
 }
+
+// ---------------------------------------------------------------------------------------
+// Second API family (inc/SparseCoo.hpp, inc/CSR.hpp, inc/prepareBlkEll.hpp, inc/splitter.hpp).
+// The library holds the fp32 instantiation; the templates exist so that reference call sites
+// such as `SparseCoo<COMPUTETYPE>`, `CSR_Matrix<COMPUTETYPE>`, `preprocess<COMPUTETYPE>`
+// (gpu_kernels.cu:1290-1292,1464) keep compiling with COMPUTETYPE = float.
+// ---------------------------------------------------------------------------------------
+#include <type_traits>
+#include <vector>
+
+template <class DType>
+struct SparseCoo {
+    static_assert(std::is_same<DType, float>::value, "libcutespmm implements the fp32 instantiation");
+    int dimY = 0, dimX = 0, nnz = 0;
+    int *rows = nullptr, *cols = nullptr;
+    DType *values = nullptr;
+    SparseCoo() = default;
+    explicit SparseCoo(const std::string &FilePath)                        // inc/SparseCoo.hpp:91-157
+    {
+        cute::check(cute_coo_read(FilePath.c_str(), &raw_), "SparseCoo");
+        sync();
+    }
+    SparseCoo(int dY, int dX, int /*nnz*/) { raw_.dimY = dY; raw_.dimX = dX; sync(); }   // :158-169
+    explicit SparseCoo(const cute_coo &owned) : raw_(owned) { sync(); }
+    void Insert_Next(int row, int col, DType val)                           // :243-248
+    {
+        if (!grown_) {   // move what a file or the library supplied into growable storage, once
+            r_.assign(raw_.rows, raw_.rows + raw_.nnz);
+            c_.assign(raw_.cols, raw_.cols + raw_.nnz);
+            v_.assign(raw_.values, raw_.values + raw_.nnz);
+            cute_coo_release(&raw_);
+        }
+        r_.push_back(row); c_.push_back(col); v_.push_back(val);
+        raw_.dimY = dimY; raw_.dimX = dimX;
+        raw_.nnz = int(r_.size());
+        rows = raw_.rows = r_.data(); cols = raw_.cols = c_.data(); values = raw_.values = v_.data();
+        nnz = raw_.nnz;
+        grown_ = true;
+    }
+    void prepare_for_cusparse() {}                                          // :250-261: the arrays are already SoA
+    void save_mtx(const std::string &path) const { cute::check(cute_coo_save_mtx(&raw_, path.c_str()), "save_mtx"); }
+    int getX() const { return dimX; }
+    int getY() const { return dimY; }
+    const cute_coo &raw() const { return raw_; }
+    ~SparseCoo() { if (!grown_) cute_coo_release(&raw_); }
+    SparseCoo(const SparseCoo &) = delete;
+    SparseCoo &operator=(const SparseCoo &) = delete;
+
+private:
+    cute_coo raw_{};
+    std::vector<int> r_, c_;
+    std::vector<DType> v_;
+    bool grown_ = false;
+    void sync() { dimY = raw_.dimY; dimX = raw_.dimX; nnz = raw_.nnz; rows = raw_.rows; cols = raw_.cols; values = raw_.values; }
+};
+
+template <class DType>
+struct CSR_Matrix {
+    static_assert(std::is_same<DType, float>::value, "libcutespmm implements the fp32 instantiation");
+    int nrows = 0, ncols = 0, nnz = 0;
+    DType *values = nullptr;
+    int *cols = nullptr, *rowPtr = nullptr;
+    int R = 0, C = 0, BCSR_nrows = 0, BCSR_ncols = 0, BCSR_nblks = 0;       // valid after to_BCSR (inc/CSR.hpp:52-60)
+    DType *BCSR_values = nullptr;
+    int *BCSR_cols = nullptr, *BCSR_rowPtr = nullptr;
+    explicit CSR_Matrix(SparseCoo<DType> &S) { coo2CSR(S); }               // inc/CSR.hpp:68-71
+    void coo2CSR(SparseCoo<DType> &S)                                       // :162-187
+    {
+        cute_csr_i32_release(&raw_);
+        cute::check(cute_coo_to_csr(&S.raw(), &raw_), "coo2CSR");
+        nrows = raw_.nrows; ncols = raw_.ncols; nnz = raw_.nnz; values = raw_.values; cols = raw_.cols; rowPtr = raw_.rowPtr;
+    }
+    template <class T> void ToDense(T *dense) const                         // :315-329
+    {
+        for (int r = 0; r < nrows; ++r)
+            for (int e = rowPtr[r]; e < rowPtr[r + 1]; ++e) dense[size_t(r) * size_t(ncols) + size_t(cols[e])] = T(values[e]);
+    }
+    int csr_count_blocks(int R_, int C_) const                              // :728-743
+    {
+        int64_t n = cute_csr_count_blocks(&raw_, R_, C_);
+        if (n < 0) throw cute::Error(int(n), "csr_count_blocks");
+        return int(n);
+    }
+    void to_BCSR(int R_, int C_)                                            // :760-810
+    {
+        cute_bcsr_release(&bcsr_);
+        cute::check(cute_csr_to_bcsr(&raw_, R_, C_, &bcsr_), "to_BCSR");
+        R = bcsr_.R; C = bcsr_.C; BCSR_nrows = bcsr_.nrows; BCSR_ncols = bcsr_.ncols; BCSR_nblks = bcsr_.nblks;
+        BCSR_values = bcsr_.values; BCSR_cols = bcsr_.cols; BCSR_rowPtr = bcsr_.rowPtr;
+    }
+    const cute_csr_i32 &raw() const { return raw_; }
+    ~CSR_Matrix() { cute_csr_i32_release(&raw_); cute_bcsr_release(&bcsr_); }
+    CSR_Matrix(const CSR_Matrix &) = delete;
+    CSR_Matrix &operator=(const CSR_Matrix &) = delete;
+
+private:
+    cute_csr_i32 raw_{};
+    cute_bcsr bcsr_{};
+};
+
+template <class DType>
+class preprocess {                                                          // inc/prepareBlkEll.hpp:15-291
+    static_assert(std::is_same<DType, float>::value, "libcutespmm implements the fp32 instantiation");
+
+public:
+    preprocess(CSR_Matrix<DType> *A_CSR, int BlockSize) : ncols_(A_CSR->ncols)
+    {
+        cute::check(cute_blocked_ell_build(&A_CSR->raw(), BlockSize, &e_), "preprocess");
+    }
+    ~preprocess() { cute_blocked_ell_release(&e_); }
+    void blockedELLToDense(DType *dense) { cute::check(cute_blocked_ell_to_dense(&e_, ncols_, dense), "blockedELLToDense"); }
+    int *get_ellColIdx() { return e_.ellColIdx; }
+    int get_ellColIdx_height() { return e_.height; }
+    int get_ellColIdx_width() { return e_.width; }
+    DType *get_ellValues() { return e_.ellValues; }
+    int get_num_blocks() { return e_.numBlocks; }
+    int get_num_elems() { return e_.numElems; }
+    preprocess(const preprocess &) = delete;
+    preprocess &operator=(const preprocess &) = delete;
+
+private:
+    cute_blocked_ell e_{};
+    int ncols_;
+};
+
+class Splitter {                                                            // inc/splitter.hpp:14-187
+public:
+    Splitter(CSR_Matrix<float> *A_CSR, int tile_size, int NNZThreshold)
+    {
+        cute::check(cute_splitter_split(&A_CSR->raw(), tile_size, NNZThreshold, &s_), "Splitter");
+        heavy_ = new SparseCoo<float>(s_.heavy);
+        light_ = new SparseCoo<float>(s_.light);
+        s_.heavy = cute_coo{};   // ownership moved into the two SparseCoo objects
+        s_.light = cute_coo{};
+    }
+    ~Splitter() { delete heavy_; delete light_; }
+    int get_total_tiles() { return s_.totalTiles; }
+    int get_num_heavy_tiles() { return s_.numHeavyTiles; }
+    int get_num_heavy_elems() { return s_.numHeavyElems; }
+    int get_num_light_tiles() { return s_.numLightTiles; }
+    int get_num_light_elems() { return s_.numLightElems; }
+    SparseCoo<float> *get_heavyMatrix() { return heavy_; }
+    SparseCoo<float> *get_lightMatrix() { return light_; }
+    Splitter(const Splitter &) = delete;
+    Splitter &operator=(const Splitter &) = delete;
+
+private:
+    cute_split s_{};
+    SparseCoo<float> *heavy_ = nullptr, *light_ = nullptr;
+};

@@ -131,3 +131,94 @@ def check_gemm(C_ref, C_test):
     assert a.shape == b.shape
     M, N = a.shape
     return float(lib().orc_check_gemm(_p(a, C.c_float), _p(b, C.c_float), C.c_uint32(M), C.c_uint32(N)))
+
+
+# ---------------------------------------------------------------- second API family
+def coo_read(path):
+    """inc/SparseCoo.hpp:91-157 -> (dimY, dimX, nnz, rows, cols, values)."""
+    dy, dx, nnz = C.c_int(), C.c_int(), C.c_int()
+    r, c, v = C.POINTER(C.c_int)(), C.POINTER(C.c_int)(), C.POINTER(C.c_float)()
+    rc = lib().orc_coo_read(os.fsencode(path), C.byref(dy), C.byref(dx), C.byref(nnz), C.byref(r), C.byref(c), C.byref(v))
+    if rc:
+        raise IOError("orc_coo_read(%s) failed: %d" % (path, rc))
+    return (dy.value, dx.value, nnz.value, _take(r, nnz.value, np.int32), _take(c, nnz.value, np.int32),
+            _take(v, nnz.value, np.float32))
+
+
+def coo_to_csr(nrows, rows, cols, vals):
+    rows, cols, vals = (np.ascontiguousarray(rows, np.int32), np.ascontiguousarray(cols, np.int32),
+                        np.ascontiguousarray(vals, np.float32))
+    rp, co, vo = np.zeros(nrows + 1, np.int32), np.zeros(len(cols), np.int32), np.zeros(len(cols), np.float32)
+    lib().orc_coo_to_csr(C.c_int(nrows), C.c_int(len(cols)), _p(rows, C.c_int), _p(cols, C.c_int), _p(vals, C.c_float),
+                         _p(rp, C.c_int), _p(co, C.c_int), _p(vo, C.c_float))
+    return rp, co, vo
+
+
+def _csr_i32(rowPtr, cols):
+    return np.ascontiguousarray(rowPtr, np.int32), np.ascontiguousarray(cols, np.int32)
+
+
+def count_blocks(nrows, ncols, rowPtr, cols, R, Cc):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    return int(lib().orc_count_blocks(C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), C.c_int(R), C.c_int(Cc)))
+
+
+def to_bcsr(nrows, ncols, rowPtr, cols, vals, R, Cc):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    vals = np.ascontiguousarray(vals, np.float32)
+    nb = count_blocks(nrows, ncols, rowPtr, cols, R, Cc)
+    brp, bc, bv = np.zeros(nrows // R + 1, np.int32), np.zeros(nb, np.int32), np.zeros(nb * R * Cc, np.float32)
+    lib().orc_to_bcsr(C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), _p(vals, C.c_float),
+                      C.c_int(R), C.c_int(Cc), _p(brp, C.c_int), _p(bc, C.c_int), _p(bv, C.c_float))
+    return brp, bc, bv
+
+
+def blocked_ell(nrows, ncols, rowPtr, cols, vals, B):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    vals = np.ascontiguousarray(vals, np.float32)
+    H, W, nb, ne = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    args = (C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), _p(vals, C.c_float), C.c_int(B))
+    lib().orc_blocked_ell(*args, C.byref(H), C.byref(W), None, None, C.byref(nb), None)
+    idx = np.zeros((H.value, max(W.value, 0)), np.int32)
+    val = np.zeros((H.value * B, W.value * B), np.float32)
+    lib().orc_blocked_ell(*args, C.byref(H), C.byref(W), _p(idx, C.c_int), _p(val, C.c_float), C.byref(nb), C.byref(ne))
+    return dict(height=H.value, width=W.value, num_blocks=nb.value, num_elems=ne.value, ellColIdx=idx, ellValues=val)
+
+
+def blocked_ell_to_dense(e, B, ncols):
+    dense = np.zeros((e["height"] * B, ncols), np.float32)
+    lib().orc_blocked_ell_to_dense(C.c_int(e["height"]), C.c_int(e["width"]), C.c_int(B), C.c_int(ncols),
+                                   _p(e["ellColIdx"], C.c_int), _p(e["ellValues"], C.c_float), _p(dense, C.c_float))
+    return dense
+
+
+def split(nrows, ncols, rowPtr, cols, tile, threshold):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    which = np.zeros(len(cols), np.uint8)
+    counters = np.zeros(5, np.int32)
+    lib().orc_split(C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), C.c_int(tile),
+                    C.c_int(threshold), _p(which, C.c_uint8), _p(counters, C.c_int))
+    return which.astype(bool), counters
+
+
+def block_stats(nrows, ncols, rowPtr, cols, B):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    nbr, nbc = (nrows + B - 1) // B, (ncols + B - 1) // B + 1
+    stats = np.zeros((nbr, nbc, 3), np.int32)
+    lib().orc_block_stats(C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), C.c_int(B), _p(stats, C.c_int))
+    return stats
+
+
+def classify(nnz, under, over, B, deviation_threshold, underload_dominance):
+    return int(lib().orc_classify(C.c_int(nnz), C.c_int(under), C.c_int(over), C.c_int(B), C.c_float(deviation_threshold),
+                                  C.c_float(underload_dominance)))
+
+
+def spmm_csr_f64(rowPtr, cols, vals, B):
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    vals, B = np.ascontiguousarray(vals, np.float64), np.ascontiguousarray(B, np.float64)
+    m, n = len(rowPtr) - 1, B.shape[1]
+    out = np.zeros((m, n), np.float64)
+    lib().orc_spmm_csr_f64(C.c_int(m), C.c_int(n), _p(rowPtr, C.c_int), _p(cols, C.c_int), _p(vals, C.c_double),
+                           _p(B, C.c_double), _p(out, C.c_double))
+    return out

@@ -1,0 +1,45 @@
+// Host-only use of the C++ mirror classes (include/cutespmm.hpp); prints one line that the
+// Python test compares with the oracle and the recorded values.  No GPU call is made.
+#include <cstdio>
+#include <vector>
+
+#include "cutespmm.hpp"
+
+int main(int argc, char **argv)
+{
+    if (argc < 2) return 2;
+    try {
+        MTX_READER reader(argv[1]);
+        HRPB hrpb(reader.M, reader.K, reader.rowPtr, reader.cols, reader.vals, /*upload=*/false);
+        SparseCoo<float> coo(argv[1]);
+        CSR_Matrix<float> csr(coo);
+        preprocess<float> ell(&csr, 16);
+        Splitter split(&csr, 16, 8);
+        csr.to_BCSR(16, 4);
+        std::vector<float> dense(size_t(ell.get_ellColIdx_height()) * 16 * size_t(csr.ncols), 0.0f), dense2(dense.size(), 0.0f);
+        ell.blockedELLToDense(dense.data());
+        csr.ToDense(dense2.data());
+        size_t diff = 0;
+        for (size_t i = 0; i < dense.size(); ++i) diff += dense[i] != dense2[i];
+        SparseCoo<float> grown(4, 4, 0);
+        grown.Insert_Next(1, 2, 3.0f);
+        grown.Insert_Next(0, 1, 2.0f);
+        CSR_Matrix<float> small(grown);
+        std::printf("M=%u K=%u nnz=%u panels=%u blocks=%u words=%llu bricks=%u bcsr=%d ell=%dx%d ellblocks=%d tiles=%d heavy=%d/%d light=%d/%d "
+                    "densediff=%zu grown=%d,%d\n",
+                    reader.M, reader.K, reader.nnz, hrpb.numRowPanels, hrpb.blockedRowPtr[hrpb.numRowPanels], hrpb.dataStructSize,
+                    hrpb.num_bricks, csr.BCSR_nblks, ell.get_ellColIdx_height(), ell.get_ellColIdx_width(), ell.get_num_blocks(),
+                    split.get_total_tiles(), split.get_num_heavy_tiles(), split.get_num_heavy_elems(), split.get_num_light_tiles(),
+                    split.get_num_light_elems(), diff, small.nnz, small.cols[0]);
+        try {
+            MTX_READER missing("/nonexistent/file.mtx");
+            return 3;
+        } catch (const cute::Error &e) {
+            if (e.status != CUTE_ERR_IO) return 4;
+        }
+    } catch (const std::exception &e) {
+        std::fprintf(stderr, "%s\n", e.what());
+        return 1;
+    }
+    return 0;
+}
