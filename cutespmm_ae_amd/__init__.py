@@ -13,7 +13,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcutespmm.so")
+LIB_PATH = os.environ.get("CUTESPMM_LIBRARY") or os.path.join(_HERE, "libcutespmm.so")
 
 # every symbol declared in include/cutespmm.h
 ABI_SYMBOLS = [
@@ -66,7 +66,8 @@ class cute_hrpb_tiled(C.Structure):
 
 class cute_tunables(C.Structure):
     _fields_ = [("path", C.c_int32), ("precision", C.c_int32), ("min_reuse", C.c_float), ("slots", C.c_uint32),
-                ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("reserved", C.c_uint32 * 1)]
+                ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("waves_per_cu", C.c_uint32), ("max_row_nnz", C.c_uint32),
+                ("reserved", C.c_uint32 * 3)]
 
 
 class cute_plan_info(C.Structure):
@@ -449,12 +450,13 @@ class SPMM_TC:
     (spmm.cu:823-839) on torch's current stream.  MatB [K,N], MatC [M,N] float32 GPU tensors."""
 
     def __init__(self, hrpb, N, path=PATH_AUTO, precision=PREC_FP32, min_reuse=0.0, slots=0, max_chunk_blocks=0,
-                 brick_groups=0, pipeline=0):
+                 brick_groups=0, pipeline=0, waves_per_cu=0, max_row_nnz=0):
         self.hrpb = hrpb
         self.M, self.K, self.N = hrpb.M, hrpb.K, int(N)
         self._plan = C.c_void_p()
         t = cute_tunables(path=path, precision=precision, min_reuse=min_reuse, slots=slots,
-                          max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline)
+                          max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline, waves_per_cu=waves_per_cu,
+                          max_row_nnz=max_row_nnz)
         _check(load_library().cute_spmm_plan_create(hrpb.upload(), self.N, C.byref(t), C.byref(self._plan)),
                "cute_spmm_plan_create")
         info = cute_plan_info()

@@ -81,6 +81,7 @@ struct cute_hrpb_dev {
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
     std::vector<uint32_t> panelCols;    // active columns per row panel
+    std::vector<uint32_t> panelMaxRow;  // longest row of each panel
 };
 
 struct cute_spmm_plan {
@@ -91,6 +92,13 @@ struct cute_spmm_plan {
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
+    uint4 *dItems = nullptr;            // persistent variant: chunks x slabs, flattened
+    uint32_t *dWaveItems = nullptr;     // persistent variant: item run of every logical wavefront
+    uint32_t persistentGroups = 0;      // work-groups of the persistent launch (multiple of 8)
+    uint32_t *dStepBlk = nullptr;       // stream variant: block id of every step
+    uint2 *dStepMeta = nullptr;         // stream variant: {panel, flags} of every step
+    uint32_t *dWaveSteps = nullptr;     // stream variant: step run of every logical wavefront
+    uint32_t streamGroups = 0, streamDepth = 0;
     uint32_t *dAtomicPanels = nullptr;
     uint32_t numAtomicPanels = 0;
     uint32_t *dRowList = nullptr;
@@ -143,8 +151,12 @@ int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
     d->brp.assign(h->blockedRowPtr, h->blockedRowPtr + h->numRowPanels + 1);
     d->panelNnz.resize(d->P);
     d->panelCols.resize(d->P);
+    d->panelMaxRow.resize(d->P);
     for (uint32_t p = 0; p < d->P; ++p) {
         d->panelNnz[p] = h->rowPtr[(p + 1) * CUTE_TM] - h->rowPtr[p * CUTE_TM];
+        uint32_t longest = 0;
+        for (uint32_t r = p * CUTE_TM; r < (p + 1) * CUTE_TM; ++r) longest = std::max(longest, h->rowPtr[r + 1] - h->rowPtr[r]);
+        d->panelMaxRow[p] = longest;
         const uint32_t nblk = d->brp[p + 1] - d->brp[p];
         uint32_t live = 0;
         if (nblk) {
@@ -190,6 +202,11 @@ void cute_spmm_plan_free(cute_spmm_plan *p)
 {
     if (!p) return;
     (void)hipFree(p->dChunks);
+    (void)hipFree(p->dItems);
+    (void)hipFree(p->dWaveItems);
+    (void)hipFree(p->dStepBlk);
+    (void)hipFree(p->dStepMeta);
+    (void)hipFree(p->dWaveSteps);
     (void)hipFree(p->dAtomicPanels);
     (void)hipFree(p->dRowList);
     delete p;
@@ -218,16 +235,22 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (t.path < CUTE_PATH_AUTO || t.path > CUTE_PATH_ROWS) return CUTE_ERR_ARG;
     if (t.precision != CUTE_PREC_FP32) return CUTE_ERR_ARG;   // the bf16x3 kernel is not built yet
     const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : 1.25f;
+    const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : 48;   // measured: longer rows serialise a lane group
 
     cute_spmm_plan *p = new cute_spmm_plan;
     p->d = d;
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    if (const char *ev = getenv("CUTE_EXP_VEC")) p->vec = std::min(p->vec, atoi(ev));   // EXPERIMENT
     p->ng = 1;   // one 16-lane column group per lane measured faster than two on every benchmark matrix
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
-    if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
+    if (t.pipeline > 4) { delete p; return CUTE_ERR_ARG; }
     p->pipeline = t.pipeline ? int(t.pipeline) : 2;
-    if (p->pipeline == 1) p->ng = 1;   // the resident variant's register budget holds one column group
+    if (p->pipeline == 1) p->ng = 1;   // the rolling variant's register budget holds one column group
+    if (p->pipeline == 4) {            // the stream variant moves 16-byte vectors through LDS
+        if (p->vec != 4) p->pipeline = 1;
+        p->ng = 1;
+    }
     const uint32_t slab = 16u * p->vec * p->ng;
     const uint32_t num_slabs = (N + slab - 1) / slab;
     // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
@@ -249,7 +272,12 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         if (nblk == 0) { rows = true; n_empty++; }
         else if (t.path == CUTE_PATH_BRICK) rows = false;
         else if (t.path == CUTE_PATH_ROWS) rows = true;
-        else rows = float(d->panelNnz[q]) < min_reuse * float(d->panelCols[q]);
+        else {
+            // Row kernel when a fetched B row serves hardly more than one nonzero of the panel
+            // (the 16-row MFMA then buys nothing) -- unless a row is so long that one lane group
+            // would serialise it: the brick kernel cuts long panels into balanced chunks.
+            rows = float(d->panelNnz[q]) < min_reuse * float(d->panelCols[q]) && d->panelMaxRow[q] <= max_row_for_rows;
+        }
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;
     }
@@ -312,9 +340,80 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             for (uint32_t r = 0; r < CUTE_TM; ++r) row_list.push_back(q * CUTE_TM + r);
 
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
+    if (rc == CUTE_OK && p->pipeline == 3 && !chunks.empty()) {
+        // persistent variant: a fixed number of wavefronts, each owning a contiguous, block-balanced
+        // run of (chunk, slab) items; XCD x owns logical wavefronts [x*W/8, (x+1)*W/8)
+        const uint32_t waves_per_cu = t.waves_per_cu ? t.waves_per_cu : 16u;
+        uint32_t groups = std::max(1u, uint32_t(c.num_cus) * waves_per_cu / cute_dev::kWavesPerGroup);
+        groups = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd;
+        const uint32_t W = groups * cute_dev::kWavesPerGroup;
+        std::vector<uint4> items;
+        items.reserve(chunks.size() * num_slabs);
+        uint64_t total = 0;
+        for (const uint4 &ck : chunks)
+            for (uint32_t sl = 0; sl < num_slabs; ++sl) {
+                items.push_back(make_uint4(ck.x, ck.y, ck.z, (ck.w & 1u) | (sl << 1)));
+                total += ck.y - ck.x;
+            }
+        std::vector<uint32_t> runs(size_t(W) + 1, uint32_t(items.size()));
+        uint64_t seen = 0;
+        uint32_t w = 0;
+        runs[0] = 0;
+        for (uint32_t i = 0; i < items.size(); ++i) {
+            // item i starts the run of every wavefront whose share begins at or before `seen`
+            while (w + 1 < W && seen >= (total * (w + 1) + W - 1) / W) runs[++w] = i;
+            seen += items[i].y - items[i].x;
+        }
+        while (w + 1 <= W) runs[++w] = uint32_t(items.size());
+        rc = upload(&p->dItems, items.data(), items.size());
+        if (rc == CUTE_OK) rc = upload(&p->dWaveItems, runs.data(), runs.size());
+        p->persistentGroups = groups;
+    }
     if (rc == CUTE_OK) rc = upload(&p->dAtomicPanels, atomic_panels.data(), atomic_panels.size());
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
+    if (rc == CUTE_OK && p->pipeline == 4 && !chunks.empty()) {
+        // stream variant: every logical wavefront gets one contiguous, block-balanced run of the
+        // flattened (chunk, slab, block) stream
+        const uint32_t depth = getenv("CUTE_EXP_DEPTH") ? uint32_t(atoi(getenv("CUTE_EXP_DEPTH"))) : 4u;   // EXPERIMENT
+        const uint32_t waves_per_cu = t.waves_per_cu ? t.waves_per_cu : 8u;
+        uint32_t groups = std::max(1u, uint32_t(c.num_cus) * waves_per_cu / cute_dev::kWavesPerGroup);
+        groups = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd;
+        const uint32_t W = groups * cute_dev::kWavesPerGroup;
+        std::vector<uint32_t> blk;
+        std::vector<uint2> meta;
+        for (const uint4 &ck : chunks)
+            for (uint32_t sl = 0; sl < num_slabs; ++sl)
+            {
+                const uint32_t common = ((ck.w & 1u) << 1) | (sl << 8);
+                const uint32_t len = (ck.y - ck.x + depth - 1) / depth * depth;   // whole ring turns
+                for (uint32_t i = 0; i < len; ++i) {
+                    const bool pad = ck.x + i >= ck.y;
+                    blk.push_back(pad ? ck.y - 1 : ck.x + i);
+                    meta.push_back(make_uint2(ck.z, common | (i + 1 == len ? 1u : 0u) | (pad ? 4u : 0u)));
+                }
+            }
+        const uint64_t total = blk.size();
+        // runs end on item boundaries where possible: cut at the first item end at or after the even share
+        std::vector<uint32_t> runs(size_t(W) + 1, uint32_t(total));
+        runs[0] = 0;
+        uint64_t pos = 0;
+        for (uint32_t w = 1; w < W; ++w) {
+            uint64_t want = std::max<uint64_t>(pos, (total * w + W - 1) / W);
+            while (want < total && want > 0 && !(meta[want - 1].y & 1u)) ++want;
+            runs[w] = uint32_t(std::min<uint64_t>(want, total));
+            pos = runs[w];
+        }
+        for (uint32_t i = 0; i < depth + 2; ++i) {     // look-ahead padding
+            blk.push_back(blk.back());
+            meta.push_back(make_uint2(meta.back().x, (meta.back().y & ~3u) | 4u));
+        }
+        rc = upload(&p->dStepBlk, blk.data(), blk.size());
+        if (rc == CUTE_OK) rc = upload(&p->dStepMeta, meta.data(), meta.size());
+        if (rc == CUTE_OK) rc = upload(&p->dWaveSteps, runs.data(), runs.size());
+        p->streamGroups = groups;
+        p->streamDepth = depth;
+    }
     p->numAtomicPanels = uint32_t(atomic_panels.size());
     p->numRows = uint32_t(row_list.size());
     p->info.N = N;
@@ -336,19 +435,48 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
 namespace {
 
+template <int DEPTH, bool FULL>
+void launch_stream(const cute_spmm_plan *p, uint32_t wpx, uint32_t zero_index, const float *dB, float *dC, hipStream_t s)
+{
+    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_stream<DEPTH, FULL>), dim3(p->streamGroups),
+                       dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dStepBlk,
+                       reinterpret_cast<const uint64_t *>(p->dStepMeta), p->dWaveSteps, wpx, p->d->dHdr, p->d->dVals,
+                       zero_index, dB, dC, p->info.N);
+}
+
 template <int VEC, int NG, bool FULL>
 void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
 {
     const uint64_t items = uint64_t(p->info.numChunks) * p->info.numSlabs;
     const uint32_t groups = uint32_t((items + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup);
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+    if (p->pipeline == 4 && VEC == 4 && NG == 1) {
+        const uint32_t wpx = p->streamGroups / cute_dev::kNumXcd * cute_dev::kWavesPerGroup;
+        const uint32_t zero_index = uint32_t(p->d->numVals);   // first float of the zero padding behind vals[]
+        switch (p->streamDepth) {
+        case 2: launch_stream<2, FULL>(p, wpx, zero_index, dB, dC, s); break;
+        case 3: launch_stream<3, FULL>(p, wpx, zero_index, dB, dC, s); break;
+        case 5: launch_stream<5, FULL>(p, wpx, zero_index, dB, dC, s); break;
+        case 6: launch_stream<6, FULL>(p, wpx, zero_index, dB, dC, s); break;
+        default: launch_stream<4, FULL>(p, wpx, zero_index, dB, dC, s); break;
+        }
+        return;
+    }
+    if (p->pipeline == 3) {
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_persistent<VEC, NG, FULL>), dim3(p->persistentGroups),
+                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dItems, p->dWaveItems,
+                           p->persistentGroups / cute_dev::kNumXcd * cute_dev::kWavesPerGroup, p->d->dHdr, p->d->dVals,
+                           dB, dC, p->info.N);
+        return;
+    }
+    static const uint32_t exp_lds = getenv("CUTE_EXP_LDS") ? uint32_t(atoi(getenv("CUTE_EXP_LDS"))) : 0u;   // EXPERIMENT
     if (p->pipeline == 1 && NG == 1)
-        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_resident<VEC, 1, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
-                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, 1, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
+                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), exp_lds, s, p->dChunks, p->info.numChunks,
                            p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
     else
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
-                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dChunks, p->info.numChunks,
+                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), exp_lds, s, p->dChunks, p->info.numChunks,
                            p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
 }
 

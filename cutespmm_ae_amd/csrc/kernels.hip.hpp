@@ -27,7 +27,10 @@ template <int VEC> __device__ __forceinline__ void vec_set(typename Vec<VEC>::ty
 template <> __device__ __forceinline__ void vec_set<1>(float &v, int, float x) { v = x; }
 
 constexpr int kWaveSize = 64;
-constexpr int kWavesPerGroup = 4;
+#ifndef CUTE_WPG
+#define CUTE_WPG 4
+#endif
+constexpr int kWavesPerGroup = CUTE_WPG;
 constexpr int kHdrWords = 32;
 constexpr int kNumXcd = 8;
 
@@ -101,7 +104,11 @@ __device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x
         for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
+#ifdef CUTE_EXPERIMENT_NO_MFMA   // timing experiment only: keeps every load alive, drops the matrix work
+                acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
+#else
                 acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
+#endif
     }
 }
 
@@ -238,12 +245,53 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
 }
 
-// Variant "resident": one operand set per wavefront and a register budget that lets eight
-// wavefronts share a SIMD, so that for short work items (a handful of blocks per panel) every
-// item of the launch is resident at once and the SIMD hides one wavefront's loads behind the
-// others' MFMAs.  Header lines still run two blocks ahead.
+// One brick's loads (A value at the lane's rank, B row segment(s)) -- the unit of the rolling
+// pipeline below.
 template <int VEC, int NG, bool FULL>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_resident(
+__device__ __forceinline__ void load_brick(BlockOperands<VEC, NG> &o, int j, const BlockHeader &hd,
+                                           const float *__restrict__ vals, const float *__restrict__ B, uint32_t N,
+                                           uint32_t col0)
+{
+    typedef typename Vec<VEC>::type V;
+    const uint32_t cols[4] = {hd.cols.x, hd.cols.y, hd.cols.z, hd.cols.w};
+    const uint64_t bm = hd.bitmap[j];
+    const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
+    o.a[j] = vals[hd.voff[j] + below];
+    o.bitmap[j] = bm;
+    const float *brow = B + size_t(cols[j]) * N + col0;
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng) {
+        if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + ng * 16 * VEC);
+        else o.b[j][ng] = V(0.0f);
+    }
+}
+
+template <int VEC, int NG, bool SKIP_EMPTY>
+__device__ __forceinline__ void mfma_brick(const BlockOperands<VEC, NG> &o, int j, f32x4 (&acc)[NG][VEC], uint32_t lane)
+{
+    if (SKIP_EMPTY && o.bitmap[j] == 0) return;     // wave-uniform: a brick made of padding columns only
+    const float a = ((o.bitmap[j] >> lane) & 1ull) ? o.a[j] : 0.0f;
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+#if defined(CUTE_EXPERIMENT_NO_MFMA)
+            acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
+#elif defined(CUTE_EXP_MFMA_BRICKS)
+            if (j < CUTE_EXP_MFMA_BRICKS) acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
+            else acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
+#else
+            acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
+#endif
+}
+
+// Variant "rolling": ONE operand set per wavefront, refilled brick by brick -- as soon as the
+// MFMAs of brick j of block i are issued, the loads of brick j of block i+1 go out into the
+// same registers.  Loads are therefore always in flight behind the MFMAs, and the register
+// budget (one operand set, one accumulator set) lets eight wavefronts share a SIMD, so a
+// launch of short panels is resident as a whole.  Padding-only bricks skip their MFMAs.
+template <int VEC, int NG, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_rolling(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
     const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
     float *__restrict__ C, uint32_t N)
@@ -259,20 +307,281 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_r
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
 
-    BlockOperands<VEC, NG> op;
-    BlockHeader hd, hn;
     uint32_t blk = it.start;
     if (blk < end) {
-        hd = load_header(hdr, blk, lane);
-        hn = load_header(hdr, min(blk + 1, end - 1), lane);
-    }
-    for (; blk < end; ++blk) {
-        load_operands<VEC, NG, FULL>(op, hd, vals, B, N, col0, lane);
-        hd = hn;
-        hn = load_header(hdr, min(blk + 2, end - 1), lane);   // clamped: the loop stays branch-free
-        mfma_block<VEC, NG>(op, acc, lane);
+        BlockOperands<VEC, NG> op;
+        BlockHeader h1, h2;
+        {
+            const BlockHeader h0 = load_header(hdr, blk, lane);
+            h1 = load_header(hdr, min(blk + 1, end - 1), lane);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_brick<VEC, NG, FULL>(op, j, h0, vals, B, N, col0);
+        }
+        // One basic block per iteration and a scheduling fence after every group, so the order
+        // "MFMAs of brick j, then the loads that refill brick j" survives instruction scheduling.
+        // Only the last block of a panel can hold padding-only bricks; it is peeled below.
+        for (; blk + 1 < end; ++blk) {       // op holds block blk, h1 the header line of blk+1
+            h2 = load_header(hdr, min(blk + 2, end - 1), lane);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                mfma_brick<VEC, NG, false>(op, j, acc, lane);
+                __builtin_amdgcn_sched_barrier(0);
+                load_brick<VEC, NG, FULL>(op, j, h1, vals, B, N, col0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            h1 = h2;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mfma_brick<VEC, NG, true>(op, j, acc, lane);
     }
     brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
+}
+
+// Variant "persistent": the launch holds a fixed number of wavefronts (a few per SIMD); each
+// walks a contiguous run of work items, items[i] = {first block, end block, panel,
+// atomic | slab << 1}.  Nothing but the first header fetch of a wavefront is exposed: header
+// lines run two blocks ahead ACROSS item boundaries (the descriptors of the next two items
+// are kept in scalar registers), and the store of one item overlaps the loads of the next.
+// wave_items[w] .. wave_items[w+1] is the run of logical wavefront w; logical ids are laid
+// out so that each XCD owns one contiguous range of items.
+template <int VEC, int NG, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32_persistent(
+    const uint4 *__restrict__ items, const uint32_t *__restrict__ wave_items, uint32_t waves_per_xcd,
+    const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
+    float *__restrict__ C, uint32_t N)
+{
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const uint32_t logical = (blockIdx.x % kNumXcd) * waves_per_xcd + (blockIdx.x / kNumXcd) * kWavesPerGroup + wave;
+    const uint32_t ib = wave_items[logical], ie = wave_items[logical + 1];
+    if (ib >= ie) return;
+
+    struct Item { uint32_t start, end, panel, flags; };
+    auto fetch = [&](uint32_t i) {
+        const uint4 q = items[min(i, ie - 1)];          // clamped: past the run the last item repeats
+        Item r;
+        r.start = __builtin_amdgcn_readfirstlane(q.x);
+        r.end = __builtin_amdgcn_readfirstlane(q.y);
+        r.panel = __builtin_amdgcn_readfirstlane(q.z);
+        r.flags = __builtin_amdgcn_readfirstlane(q.w);
+        return r;
+    };
+    Item cur = fetch(ib), nx1 = fetch(ib + 1), nx2 = fetch(ib + 2);
+    // block id `ahead` (1 or 2) steps after block `blk` of the current item, in stream order
+    auto lookahead = [&](uint32_t blk, uint32_t ahead) {
+        if (blk + ahead < cur.end) return blk + ahead;
+        const uint32_t over = blk + ahead - cur.end, len1 = nx1.end - nx1.start;
+        return over < len1 ? nx1.start + over : nx2.start + (over - len1);
+    };
+
+    f32x4 acc[NG][VEC];
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
+
+    // Rolling refill across item boundaries: `op` holds the current block of the stream, h1 the
+    // header line of the next block of the stream (possibly the first block of the next item,
+    // whose slab -- hence B column offset -- may differ), h2 the one after that.
+    auto col0_of = [&](const Item &q) { return (q.flags >> 1) * (16u * VEC * NG) + (lane & 15u) * VEC; };
+    BlockOperands<VEC, NG> op;
+    uint32_t item = ib, blk = cur.start;
+    BlockHeader h1, h2;
+    {
+        const BlockHeader h0 = load_header(hdr, blk, lane);
+        h1 = load_header(hdr, lookahead(blk, 1), lane);
+        const uint32_t c0 = col0_of(cur);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_brick<VEC, NG, FULL>(op, j, h0, vals, B, N, c0);
+    }
+    while (true) {
+        const bool last_of_item = blk + 1 == cur.end;
+        const uint32_t col0_next = last_of_item ? col0_of(nx1) : col0_of(cur);
+        const uint32_t blk_next = lookahead(blk, 1);
+        h2 = load_header(hdr, lookahead(blk, 2), lane);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            mfma_brick<VEC, NG, false>(op, j, acc, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            load_brick<VEC, NG, FULL>(op, j, h1, vals, B, N, col0_next);   // past the run: a harmless re-read
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        h1 = h2;
+        if (last_of_item) {
+            BrickItem done;
+            done.panel = cur.panel;
+            done.atomic = cur.flags & 1u;
+            done.col0 = col0_of(cur);
+            brick_store<VEC, NG, FULL>(done, acc, C, N, lane);
+#pragma unroll
+            for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
+            if (++item == ie) break;
+            cur = nx1;
+            nx1 = nx2;
+            nx2 = fetch(item + 2);
+        }
+        blk = blk_next;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Variant "stream": persistent wavefronts, each with a ring of DEPTH operand sets in registers.
+//
+// In the variants above every wavefront of a launch asks for its first operands at the same
+// moment and writes its C tile at the same moment, so the matrix pipes idle while the first
+// loads and the last stores are served.  Here a few wavefronts per SIMD each walk a long run
+// of blocks: the loads of block t+DEPTH are issued as soon as the MFMAs of block t have been
+// issued, C tiles are written (without waiting for them) while the following blocks are already
+// in flight, and the matrix pipe starts as soon as the first block of a run has landed.
+//
+// The host flattens the work into one stream of blocks per wavefront:
+//   step_blk[t]   block id
+//   step_meta[t]  low word: row panel; high word: flags
+//                 flags bit0 last step of its item (store C afterwards),
+//                       bit1 combine through atomics,
+//                       bit2 padding step (items are padded to a whole number of ring turns),
+//                       bits 8.. slab index (64 columns per slab)
+// wave_steps[w] .. wave_steps[w+1] is the run of logical wavefront w (XCD-contiguous ids); runs
+// end on item boundaries.  Both step arrays are padded by DEPTH+2 repeats of the last step, so
+// look-ahead never leaves them.
+//
+// Header lines are wave-uniform and are fetched with scalar loads only; every block issues
+// exactly eight vector loads (4 A, 4 B), also past the end of a run (there the B part is pointed
+// at the zero pad behind the values), so the number of loads in flight behind any operand set
+// is a compile-time constant and the waits never drain the ring.
+// ---------------------------------------------------------------------------------------
+struct ScalarHeader {        // a whole header line in scalar registers
+    uint32_t cols[16];
+    uint64_t bitmap[4];
+    uint32_t voff[4];
+};
+
+__device__ __forceinline__ ScalarHeader load_scalar_header(const uint32_t *__restrict__ hdr, uint32_t blk)
+{
+    const uint32_t *h = hdr + size_t(blk) * kHdrWords;
+    ScalarHeader r;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r.cols[i] = h[i];
+    const uint64_t *bm = reinterpret_cast<const uint64_t *>(h + 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.bitmap[j] = bm[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.voff[j] = h[24 + j];
+    return r;
+}
+
+struct StreamOperands {      // one block: masked A values and B row segments of its four bricks
+    float a[4];
+    f32x4 b[4];
+};
+
+// keep == 0 (padding step, or a step past the end of the run) turns every A value into the stored zero.
+__device__ __forceinline__ void stream_issue(StreamOperands &o, const ScalarHeader &h, const float *__restrict__ vals,
+                                             uint32_t keep, uint32_t zero_index, const float *__restrict__ B, uint32_t N,
+                                             uint32_t col, uint32_t lane)
+{
+    const uint32_t g = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        // column of lane group g in brick j: header word g*4 + j
+        const uint32_t c01 = g == 0 ? h.cols[j] : h.cols[4 + j];
+        const uint32_t c23 = g == 2 ? h.cols[8 + j] : h.cols[12 + j];
+        const uint32_t colj = g < 2 ? c01 : c23;
+        const uint64_t bm = h.bitmap[j] & (uint64_t(keep) | (uint64_t(keep) << 32));
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
+        // lanes whose bit is clear read a stored zero, so the register holds the masked A operand
+        const uint32_t aidx = ((bm >> lane) & 1ull) ? h.voff[j] + below : zero_index;
+        o.a[j] = vals[aidx];
+        o.b[j] = *reinterpret_cast<const f32x4 *>(B + size_t(colj) * N + col);
+    }
+}
+
+template <int DEPTH, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32_stream(
+    const uint32_t *__restrict__ step_blk, const uint64_t *__restrict__ step_meta, const uint32_t *__restrict__ wave_steps,
+    uint32_t waves_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ vals, uint32_t zero_index,
+    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+{
+    static_assert(DEPTH >= 2 && DEPTH <= 6, "ring depth");
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const uint32_t logical = (blockIdx.x % kNumXcd) * waves_per_xcd + (blockIdx.x / kNumXcd) * kWavesPerGroup + wave;
+    const uint32_t t0 = wave_steps[logical], t1 = wave_steps[logical + 1];
+    if (t0 >= t1) return;
+    const uint32_t lane_col = (lane & 15u) * 4u;
+    auto column_of = [&](uint32_t flags) {
+        const uint32_t c = (flags >> 8) * 64u + lane_col;
+        return FULL ? c : min(c, N - 4u);          // ragged tail: re-read the last full vector, masked at the store
+    };
+    const float *zeros = vals + zero_index;
+
+    StreamOperands ring[DEPTH];
+    // prologue: fill the ring
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) {
+        const ScalarHeader h = load_scalar_header(hdr, step_blk[t0 + i]);
+        const uint32_t f = uint32_t(step_meta[t0 + i] >> 32);
+        const bool live = !(f & 4u);              // a run holds at least one whole item, i.e. DEPTH steps
+        stream_issue(ring[i], h, vals, live ? 0xffffffffu : 0u, zero_index, live ? B : zeros, live ? N : 0u,
+                     live ? column_of(f) : lane_col, lane);
+    }
+    // scalar look-ahead: header of step t+DEPTH (used at the end of step t), block id of t+DEPTH+1
+    ScalarHeader h_issue = load_scalar_header(hdr, step_blk[t0 + DEPTH]);
+    uint32_t blk_ahead = step_blk[t0 + DEPTH + 1];
+    uint32_t flags_issue = uint32_t(step_meta[t0 + DEPTH] >> 32);
+
+    uint32_t t = t0;
+    do {   // one item: a whole number of ring turns that ends with a C tile
+        f32x4 acc[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[v] = f32x4(0.0f);
+        uint64_t meta;
+        do {   // one ring turn
+#pragma unroll
+            for (int s = 0; s < DEPTH; ++s) {
+                StreamOperands &o = ring[s];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        acc[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[j], o.b[j][v], acc[v], 0, 0, 0);
+                // refill the set just consumed with block t+s+DEPTH, then advance the scalar look-ahead
+                {
+                    const bool live = !(flags_issue & 4u) && t + s + DEPTH < t1;
+                    stream_issue(o, h_issue, vals, live ? 0xffffffffu : 0u, zero_index, live ? B : zeros, live ? N : 0u,
+                                 live ? column_of(flags_issue) : lane_col, lane);
+                }
+                h_issue = load_scalar_header(hdr, blk_ahead);
+                flags_issue = uint32_t(step_meta[t + s + DEPTH + 1] >> 32);
+                blk_ahead = step_blk[t + s + DEPTH + 2];
+            }
+            meta = step_meta[t + DEPTH - 1];
+            t += DEPTH;
+        } while (!(uint32_t(meta >> 32) & 1u));
+        // end of the item: write its C tile; the stores are not waited for
+        const uint32_t flags = uint32_t(meta >> 32);
+        const uint32_t c = (flags >> 8) * 64u + lane_col;
+        if (FULL || c < N) {
+            const uint32_t row0 = uint32_t(meta) * 16u + (lane >> 4) * 4u;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float *dst = C + size_t(row0 + r) * N + c;
+                if (flags & 2u) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) unsafeAtomicAdd(dst + v, acc[v][r]);
+                } else {
+                    f32x4 out;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) out[v] = acc[v][r];
+                    *reinterpret_cast<f32x4 *>(dst) = out;
+                }
+            }
+        }
+    } while (t < t1);
 }
 
 // Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).

@@ -256,8 +256,10 @@ typedef struct cute_tunables {
     uint32_t slots;            /* resident work items assumed by the partition; 0: derive from device */
     uint32_t max_chunk_blocks; /* upper bound on blocks per work item; 0: none            */
     uint32_t brick_groups;     /* 16-lane column groups per lane in the brick kernel (1 or 2); 0: default */
-    uint32_t pipeline;         /* brick kernel variant: 1 resident (one operand set, 8 wavefronts/SIMD), 2 pipelined; 0: default */
-    uint32_t reserved[1];
+    uint32_t pipeline;         /* brick kernel variant: 1 resident, 2 pipelined, 3 persistent; 0: default          */
+    uint32_t waves_per_cu;     /* persistent variant: wavefronts launched per CU; 0: default                      */
+    uint32_t max_row_nnz;      /* AUTO: panels holding a row longer than this stay on the brick kernel; 0: default  */
+    uint32_t reserved[3];
 } cute_tunables;
 
 typedef struct cute_plan_info {
