@@ -21,6 +21,7 @@ ABI_SYMBOLS = [
     "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
+    "cute_quad_build", "cute_quad_release",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
@@ -64,9 +65,14 @@ class cute_hrpb_tiled(C.Structure):
                 ("numVals", C.c_uint64), ("blockedRowPtr", u32p), ("hdr", u32p), ("vals", f32p)]
 
 
+class cute_quad_lists(C.Structure):
+    _fields_ = [("M", C.c_uint32), ("K", C.c_uint32), ("numRowPanels", C.c_uint32), ("numGroups", C.c_uint64),
+                ("groupPtr", u32p), ("cols", u32p), ("vals", f32p)]
+
+
 class cute_tunables(C.Structure):
     _fields_ = [("path", C.c_int32), ("precision", C.c_int32), ("min_reuse", C.c_float), ("slots", C.c_uint32),
-                ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("waves_per_cu", C.c_uint32), ("max_row_nnz", C.c_uint32),
+                ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("mfma_shape", C.c_uint32), ("max_row_nnz", C.c_uint32),
                 ("reserved", C.c_uint32 * 3)]
 
 
@@ -143,6 +149,9 @@ def load_library():
     lib.cute_hrpb_retile.argtypes = [C.POINTER(cute_hrpb_host), C.POINTER(cute_hrpb_tiled)]
     lib.cute_hrpb_untile.argtypes = [C.POINTER(cute_hrpb_tiled), C.POINTER(cute_hrpb_host)]
     lib.cute_hrpb_tiled_release.argtypes = [C.POINTER(cute_hrpb_tiled)]
+    lib.cute_quad_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_quad_lists)]
+    lib.cute_quad_release.argtypes = [C.POINTER(cute_quad_lists)]
+    lib.cute_quad_release.restype = None
     lib.cute_partition.restype = C.c_int64
     lib.cute_partition.argtypes = [C.c_uint32, u32p, C.c_uint32, C.c_uint32, u32p, C.c_uint64]
     lib.cute_check_gemm_correctness.restype = C.c_float
@@ -439,6 +448,23 @@ def _dev_ptr(t):
     return C.c_void_p(t.data_ptr())
 
 
+def quad_lists(M, K, rowPtr, cols, vals):
+    """Host copy of the 4x4x1 MFMA kernel's layout built from a CSR matrix:
+    dict(groupPtr[P+1], cols[G,16], vals[G,64])."""
+    rowPtr = np.ascontiguousarray(rowPtr, np.uint32)
+    cols = np.ascontiguousarray(cols, np.uint32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    q = cute_quad_lists()
+    _check(load_library().cute_quad_build(int(M), int(K), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p),
+                                          C.byref(q)), "cute_quad_build")
+    out = dict(numGroups=int(q.numGroups),
+               groupPtr=_view(q.groupPtr, q.numRowPanels + 1, np.uint32).copy(),
+               cols=_view(q.cols, q.numGroups * 16, np.uint32).reshape(-1, 16).copy(),
+               vals=_view(q.vals, q.numGroups * 64, np.float32).reshape(-1, 64).copy())
+    load_library().cute_quad_release(C.byref(q))
+    return out
+
+
 def _stream_ptr(stream):
     import torch
     s = stream if stream is not None else torch.cuda.current_stream()
@@ -450,12 +476,12 @@ class SPMM_TC:
     (spmm.cu:823-839) on torch's current stream.  MatB [K,N], MatC [M,N] float32 GPU tensors."""
 
     def __init__(self, hrpb, N, path=PATH_AUTO, precision=PREC_FP32, min_reuse=0.0, slots=0, max_chunk_blocks=0,
-                 brick_groups=0, pipeline=0, waves_per_cu=0, max_row_nnz=0):
+                 brick_groups=0, pipeline=0, mfma_shape=0, max_row_nnz=0):
         self.hrpb = hrpb
         self.M, self.K, self.N = hrpb.M, hrpb.K, int(N)
         self._plan = C.c_void_p()
         t = cute_tunables(path=path, precision=precision, min_reuse=min_reuse, slots=slots,
-                          max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline, waves_per_cu=waves_per_cu,
+                          max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline, mfma_shape=mfma_shape,
                           max_row_nnz=max_row_nnz)
         _check(load_library().cute_spmm_plan_create(hrpb.upload(), self.N, C.byref(t), C.byref(self._plan)),
                "cute_spmm_plan_create")

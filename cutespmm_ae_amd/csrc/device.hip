@@ -78,7 +78,11 @@ struct cute_hrpb_dev {
     float *dVals = nullptr;
     uint32_t *dRowPtr = nullptr, *dCols = nullptr;
     float *dCsrVals = nullptr;
+    uint32_t *dQCols = nullptr;         // quad lists: 16 columns per group
+    float *dQVals = nullptr;            // quad lists: 64 values per group
+    uint64_t numGroups = 0;
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
+    std::vector<uint32_t> qgp;          // host copy of the quad lists' groupPtr
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
     std::vector<uint32_t> panelCols;    // active columns per row panel
     std::vector<uint32_t> panelMaxRow;  // longest row of each panel
@@ -88,17 +92,11 @@ struct cute_spmm_plan {
     const cute_hrpb_dev *d = nullptr;
     cute_plan_info info{};
     int vec = 4, ng = 1;                // brick kernel shape
-    int pipeline = 2;                   // 1: resident variant, 2: pipelined variant
+    int pipeline = 1;                   // 1: rolling variant, 2: pipelined variant
+    int shape = 2;                      // MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
-    uint4 *dItems = nullptr;            // persistent variant: chunks x slabs, flattened
-    uint32_t *dWaveItems = nullptr;     // persistent variant: item run of every logical wavefront
-    uint32_t persistentGroups = 0;      // work-groups of the persistent launch (multiple of 8)
-    uint32_t *dStepBlk = nullptr;       // stream variant: block id of every step
-    uint2 *dStepMeta = nullptr;         // stream variant: {panel, flags} of every step
-    uint32_t *dWaveSteps = nullptr;     // stream variant: step run of every logical wavefront
-    uint32_t streamGroups = 0, streamDepth = 0;
     uint32_t *dAtomicPanels = nullptr;
     uint32_t numAtomicPanels = 0;
     uint32_t *dRowList = nullptr;
@@ -127,6 +125,8 @@ void cute_hrpb_dev_free(cute_hrpb_dev *d)
     (void)hipFree(d->dRowPtr);
     (void)hipFree(d->dCols);
     (void)hipFree(d->dCsrVals);
+    (void)hipFree(d->dQCols);
+    (void)hipFree(d->dQVals);
     delete d;
 }
 
@@ -184,6 +184,18 @@ int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
     d->bytes = uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + t.numVals * 4 + (uint64_t(h->M) + 1) * 4 +
                uint64_t(h->nnz) * 8;
     cute_hrpb_tiled_release(&t);
+    if (rc == CUTE_OK) {
+        cute_quad_lists ql;
+        rc = cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
+        if (rc == CUTE_OK) {
+            d->numGroups = ql.numGroups;
+            d->qgp.assign(ql.groupPtr, ql.groupPtr + ql.numRowPanels + 1);
+            rc = upload(&d->dQCols, ql.cols, ql.numGroups * 16);
+            if (rc == CUTE_OK) rc = upload(&d->dQVals, ql.vals, ql.numGroups * 64);
+            d->bytes += ql.numGroups * (16 + 64) * 4;
+            cute_quad_release(&ql);
+        }
+    }
     if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
     *out = d;
     return CUTE_OK;
@@ -202,11 +214,6 @@ void cute_spmm_plan_free(cute_spmm_plan *p)
 {
     if (!p) return;
     (void)hipFree(p->dChunks);
-    (void)hipFree(p->dItems);
-    (void)hipFree(p->dWaveItems);
-    (void)hipFree(p->dStepBlk);
-    (void)hipFree(p->dStepMeta);
-    (void)hipFree(p->dWaveSteps);
     (void)hipFree(p->dAtomicPanels);
     (void)hipFree(p->dRowList);
     delete p;
@@ -239,30 +246,6 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
     cute_spmm_plan *p = new cute_spmm_plan;
     p->d = d;
-    // brick kernel shape
-    p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
-    if (const char *ev = getenv("CUTE_EXP_VEC")) p->vec = std::min(p->vec, atoi(ev));   // EXPERIMENT
-    p->ng = 1;   // one 16-lane column group per lane measured faster than two on every benchmark matrix
-    if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
-    if (t.pipeline > 4) { delete p; return CUTE_ERR_ARG; }
-    p->pipeline = t.pipeline ? int(t.pipeline) : 2;
-    if (p->pipeline == 1) p->ng = 1;   // the rolling variant's register budget holds one column group
-    if (p->pipeline == 4) {            // the stream variant moves 16-byte vectors through LDS
-        if (p->vec != 4) p->pipeline = 1;
-        p->ng = 1;
-    }
-    const uint32_t slab = 16u * p->vec * p->ng;
-    const uint32_t num_slabs = (N + slab - 1) / slab;
-    // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
-    p->rows_vec = p->vec;
-    {
-        uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
-        while ((1u << logl) < need && logl < 6) ++logl;
-        p->rows_logl = int(logl);
-        const uint32_t w = (1u << logl) * p->rows_vec;
-        p->rows_slabs = (N + w - 1) / w;
-    }
-
     // classify panels
     std::vector<uint8_t> to_rows(d->P, 0);
     uint32_t n_brick = 0, n_rows = 0, n_empty = 0;
@@ -282,29 +265,67 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         if (nblk) (rows ? n_rows : n_brick)++;
     }
 
+    // brick kernel shape
+    p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    p->ng = 1;   // one 16-lane column group per lane measured faster than two on every benchmark matrix
+    if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
+    if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
+    // the rolling variant addresses B and the values with 32-bit byte offsets (24 x 24-bit product)
+    const bool offsets_fit = d->K < (1u << 24) && d->M < (1u << 24) && uint64_t(N) * 4u < (1u << 24) &&
+                             uint64_t(d->K) * N * 4u <= 0xffffffffull && uint64_t(d->M + 16u) * N * 4u <= 0xffffffffull &&
+                             (d->numVals + 64u) * 4u <= 0xffffffffull;
+    p->pipeline = t.pipeline ? int(t.pipeline) : 1;
+    if (p->pipeline == 1 && !offsets_fit) p->pipeline = 2;
+    if (t.mfma_shape > 2) { delete p; return CUTE_ERR_ARG; }
+    if (t.mfma_shape) p->shape = int(t.mfma_shape);
+    else {
+        // A 16x4 brick costs the same matrix time however few nonzeros it holds; the quad lists
+        // only pay for occupied (4-row group, column) pairs but fetch a B row once per row group
+        // instead of once per panel.  Measured break-even: about 14 nonzeros per brick.
+        uint64_t nz = 0, bricks = 0;
+        for (uint32_t q = 0; q < d->P; ++q)
+            if (!to_rows[q]) { nz += d->panelNnz[q]; bricks += (d->panelCols[q] + 3u) / 4u; }
+        p->shape = nz < 14u * bricks ? 2 : 1;
+    }
+    if (p->shape == 2 && !(offsets_fit && d->numGroups * 64u * 4u <= 0xffffffffull)) p->shape = 1;
+    const uint32_t slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
+    const uint32_t num_slabs = (N + slab - 1) / slab;
+    if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
+    // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
+    p->rows_vec = p->vec;
+    {
+        uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
+        while ((1u << logl) < need && logl < 6) ++logl;
+        p->rows_logl = int(logl);
+        const uint32_t w = (1u << logl) * p->rows_vec;
+        p->rows_slabs = (N + w - 1) / w;
+    }
+
     // chunk list for the brick kernel.  With t.slots set, the reference arithmetic
     // (spmm.cu:776-812) decides which panels are cut; its default there would cut every panel
     // that is one block above the (floored) mean as soon as the device holds all work items
     // at once, which is the normal case on 256 CUs.  The default policy therefore cuts only
     // outliers: a panel is split when it is more than twice as long as the per-item share
     // of the whole job (and at least 8 blocks), into pieces of about that share.
+    // work units along a panel: 16-column blocks for the brick kernel, groups for the quad kernel
+    const std::vector<uint32_t> &unit = p->shape == 2 ? d->qgp : d->brp;
     const uint32_t resident = uint32_t(c.num_cus) * 4u * 8u;   // 4 SIMDs x 8 wavefronts per CU
     const uint32_t slots = t.slots ? t.slots : resident;
     std::vector<uint32_t> quads;
     if (t.slots) {
-        int64_t n = cute_partition(d->P, d->brp.data(), num_slabs, slots, nullptr, 0);
+        int64_t n = cute_partition(d->P, unit.data(), num_slabs, slots, nullptr, 0);
         if (n < 0) { delete p; return int(n); }
         quads.resize(uint64_t(n) * 4);
-        cute_partition(d->P, d->brp.data(), num_slabs, slots, quads.data(), uint64_t(n));
+        cute_partition(d->P, unit.data(), num_slabs, slots, quads.data(), uint64_t(n));
     } else {
         uint64_t work = 0;
         for (uint32_t q = 0; q < d->P; ++q)
-            if (!to_rows[q]) work += d->brp[q + 1] - d->brp[q];
+            if (!to_rows[q]) work += unit[q + 1] - unit[q];
         const uint64_t mean = n_brick ? (work + n_brick - 1) / n_brick : 1;
         const uint64_t share = (work * num_slabs + resident - 1) / resident;
         const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, mean), 8));
         for (uint32_t q = 0; q < d->P; ++q) {
-            const uint32_t s = d->brp[q], e = d->brp[q + 1];
+            const uint32_t s = unit[q], e = unit[q + 1];
             if (s == e || to_rows[q]) continue;
             const uint32_t nblk = e - s;
             if (nblk <= 2 * target) {
@@ -340,80 +361,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             for (uint32_t r = 0; r < CUTE_TM; ++r) row_list.push_back(q * CUTE_TM + r);
 
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
-    if (rc == CUTE_OK && p->pipeline == 3 && !chunks.empty()) {
-        // persistent variant: a fixed number of wavefronts, each owning a contiguous, block-balanced
-        // run of (chunk, slab) items; XCD x owns logical wavefronts [x*W/8, (x+1)*W/8)
-        const uint32_t waves_per_cu = t.waves_per_cu ? t.waves_per_cu : 16u;
-        uint32_t groups = std::max(1u, uint32_t(c.num_cus) * waves_per_cu / cute_dev::kWavesPerGroup);
-        groups = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd;
-        const uint32_t W = groups * cute_dev::kWavesPerGroup;
-        std::vector<uint4> items;
-        items.reserve(chunks.size() * num_slabs);
-        uint64_t total = 0;
-        for (const uint4 &ck : chunks)
-            for (uint32_t sl = 0; sl < num_slabs; ++sl) {
-                items.push_back(make_uint4(ck.x, ck.y, ck.z, (ck.w & 1u) | (sl << 1)));
-                total += ck.y - ck.x;
-            }
-        std::vector<uint32_t> runs(size_t(W) + 1, uint32_t(items.size()));
-        uint64_t seen = 0;
-        uint32_t w = 0;
-        runs[0] = 0;
-        for (uint32_t i = 0; i < items.size(); ++i) {
-            // item i starts the run of every wavefront whose share begins at or before `seen`
-            while (w + 1 < W && seen >= (total * (w + 1) + W - 1) / W) runs[++w] = i;
-            seen += items[i].y - items[i].x;
-        }
-        while (w + 1 <= W) runs[++w] = uint32_t(items.size());
-        rc = upload(&p->dItems, items.data(), items.size());
-        if (rc == CUTE_OK) rc = upload(&p->dWaveItems, runs.data(), runs.size());
-        p->persistentGroups = groups;
-    }
     if (rc == CUTE_OK) rc = upload(&p->dAtomicPanels, atomic_panels.data(), atomic_panels.size());
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
-    if (rc == CUTE_OK && p->pipeline == 4 && !chunks.empty()) {
-        // stream variant: every logical wavefront gets one contiguous, block-balanced run of the
-        // flattened (chunk, slab, block) stream
-        const uint32_t depth = getenv("CUTE_EXP_DEPTH") ? uint32_t(atoi(getenv("CUTE_EXP_DEPTH"))) : 4u;   // EXPERIMENT
-        const uint32_t waves_per_cu = t.waves_per_cu ? t.waves_per_cu : 8u;
-        uint32_t groups = std::max(1u, uint32_t(c.num_cus) * waves_per_cu / cute_dev::kWavesPerGroup);
-        groups = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd;
-        const uint32_t W = groups * cute_dev::kWavesPerGroup;
-        std::vector<uint32_t> blk;
-        std::vector<uint2> meta;
-        for (const uint4 &ck : chunks)
-            for (uint32_t sl = 0; sl < num_slabs; ++sl)
-            {
-                const uint32_t common = ((ck.w & 1u) << 1) | (sl << 8);
-                const uint32_t len = (ck.y - ck.x + depth - 1) / depth * depth;   // whole ring turns
-                for (uint32_t i = 0; i < len; ++i) {
-                    const bool pad = ck.x + i >= ck.y;
-                    blk.push_back(pad ? ck.y - 1 : ck.x + i);
-                    meta.push_back(make_uint2(ck.z, common | (i + 1 == len ? 1u : 0u) | (pad ? 4u : 0u)));
-                }
-            }
-        const uint64_t total = blk.size();
-        // runs end on item boundaries where possible: cut at the first item end at or after the even share
-        std::vector<uint32_t> runs(size_t(W) + 1, uint32_t(total));
-        runs[0] = 0;
-        uint64_t pos = 0;
-        for (uint32_t w = 1; w < W; ++w) {
-            uint64_t want = std::max<uint64_t>(pos, (total * w + W - 1) / W);
-            while (want < total && want > 0 && !(meta[want - 1].y & 1u)) ++want;
-            runs[w] = uint32_t(std::min<uint64_t>(want, total));
-            pos = runs[w];
-        }
-        for (uint32_t i = 0; i < depth + 2; ++i) {     // look-ahead padding
-            blk.push_back(blk.back());
-            meta.push_back(make_uint2(meta.back().x, (meta.back().y & ~3u) | 4u));
-        }
-        rc = upload(&p->dStepBlk, blk.data(), blk.size());
-        if (rc == CUTE_OK) rc = upload(&p->dStepMeta, meta.data(), meta.size());
-        if (rc == CUTE_OK) rc = upload(&p->dWaveSteps, runs.data(), runs.size());
-        p->streamGroups = groups;
-        p->streamDepth = depth;
-    }
     p->numAtomicPanels = uint32_t(atomic_panels.size());
     p->numRows = uint32_t(row_list.size());
     p->info.N = N;
@@ -435,49 +385,18 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
 namespace {
 
-template <int DEPTH, bool FULL>
-void launch_stream(const cute_spmm_plan *p, uint32_t wpx, uint32_t zero_index, const float *dB, float *dC, hipStream_t s)
-{
-    hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_stream<DEPTH, FULL>), dim3(p->streamGroups),
-                       dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dStepBlk,
-                       reinterpret_cast<const uint64_t *>(p->dStepMeta), p->dWaveSteps, wpx, p->d->dHdr, p->d->dVals,
-                       zero_index, dB, dC, p->info.N);
-}
-
 template <int VEC, int NG, bool FULL>
 void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
 {
-    const uint64_t items = uint64_t(p->info.numChunks) * p->info.numSlabs;
-    const uint32_t groups = uint32_t((items + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup);
+    const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
-    if (p->pipeline == 4 && VEC == 4 && NG == 1) {
-        const uint32_t wpx = p->streamGroups / cute_dev::kNumXcd * cute_dev::kWavesPerGroup;
-        const uint32_t zero_index = uint32_t(p->d->numVals);   // first float of the zero padding behind vals[]
-        switch (p->streamDepth) {
-        case 2: launch_stream<2, FULL>(p, wpx, zero_index, dB, dC, s); break;
-        case 3: launch_stream<3, FULL>(p, wpx, zero_index, dB, dC, s); break;
-        case 5: launch_stream<5, FULL>(p, wpx, zero_index, dB, dC, s); break;
-        case 6: launch_stream<6, FULL>(p, wpx, zero_index, dB, dC, s); break;
-        default: launch_stream<4, FULL>(p, wpx, zero_index, dB, dC, s); break;
-        }
-        return;
-    }
-    if (p->pipeline == 3) {
-        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_persistent<VEC, NG, FULL>), dim3(p->persistentGroups),
-                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), 0, s, p->dItems, p->dWaveItems,
-                           p->persistentGroups / cute_dev::kNumXcd * cute_dev::kWavesPerGroup, p->d->dHdr, p->d->dVals,
-                           dB, dC, p->info.N);
-        return;
-    }
-    static const uint32_t exp_lds = getenv("CUTE_EXP_LDS") ? uint32_t(atoi(getenv("CUTE_EXP_LDS"))) : 0u;   // EXPERIMENT
-    if (p->pipeline == 1 && NG == 1)
-        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, 1, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
-                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), exp_lds, s, p->dChunks, p->info.numChunks,
-                           p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+    const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
+    if (p->pipeline == 1)
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, NG, FULL>), grid, block, 0, s, p->dChunks,
+                           p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, p->info.N);
     else
-        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), dim3(per_xcd * cute_dev::kNumXcd),
-                           dim3(cute_dev::kWaveSize * cute_dev::kWavesPerGroup), exp_lds, s, p->dChunks, p->info.numChunks,
-                           p->info.numSlabs, per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+        hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), grid, block, 0, s, p->dChunks, p->info.numChunks,
+                           per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
 }
 
 template <int VEC, int NG>
@@ -590,7 +509,17 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         hipLaunchKernelGGL(cute_dev::zero_panels, dim3(p->numAtomicPanels), dim3(256), 0, s, p->dAtomicPanels,
                            p->numAtomicPanels, dC, N);
     }
-    if (p->info.numChunks) {
+    if (p->info.numChunks && p->shape == 2) {
+        const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
+        const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+        const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
+        if (N % 64u == 0)
+            hipLaunchKernelGGL(cute_dev::hrpb_quad_f32<true>, grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,
+                               p->d->dQCols, p->d->dQVals, dB, dC, N);
+        else
+            hipLaunchKernelGGL(cute_dev::hrpb_quad_f32<false>, grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,
+                               p->d->dQCols, p->d->dQVals, dB, dC, N);
+    } else if (p->info.numChunks) {
         if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
         else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);
         else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, s);

@@ -1,0 +1,120 @@
+// Quad lists: the device layout of the 4x4x1 MFMA kernel.
+//
+// The canonical HRPB format (reference data.cu:97-246) groups the active columns of a 16-row
+// panel into 16x4 bricks, which fit a 16-row matrix instruction.  On gfx950 the fp32 matrix
+// instructions all run at the same rate and share the SIMD's issue stream with vector work, so
+// what counts is how many of them a panel needs.  v_mfma_f32_4x4x1_16B_f32 with an A broadcast
+// multiplies ONE column of FOUR rows into 64 output columns, so a panel only pays for the
+// (4-row group, column) pairs that hold a nonzero: each of the four row groups of a panel gets
+// its own sorted list of active columns, the four lists advance in lockstep (padded to the
+// longest), and 16 pairs -- four steps of the four groups -- form one "group" of the layout:
+//   cols[g*16 + 4*s + rg]          column of row group rg at step s of group g
+//   vals[g*64 + 4*(4*s + rg) + i]  value of row 4*rg+i in that column (0 if absent)
+// vals is exactly the A register of the kernel: lane 4*p+i, pair p = 4*s+rg.
+#include "common.hpp"
+#include "../../include/cutespmm.h"
+
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+// Walks the merged, duplicate-free column list of rows [r0, r0+4) of a CSR matrix.  emit(col, v)
+// receives each column once with the four row values (0 where a row has no entry there).
+template <class Emit>
+uint32_t merge_row_group(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t r0, Emit emit)
+{
+    uint32_t cur[4], end[4];
+    for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t r = r0 + i;
+        cur[i] = r < M ? rowPtr[r] : 0;
+        end[i] = r < M ? rowPtr[r + 1] : 0;
+    }
+    uint32_t count = 0;
+    for (;;) {
+        uint32_t col = UINT32_MAX;
+        bool any = false;
+        for (uint32_t i = 0; i < 4; ++i)
+            if (cur[i] < end[i]) { col = std::min(col, cols[cur[i]]); any = true; }
+        if (!any) break;
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t i = 0; i < 4; ++i)
+            // a duplicated (row, column) entry keeps its last value, as a dense scatter would
+            while (cur[i] < end[i] && cols[cur[i]] == col) v[i] = vals[cur[i]++];
+        emit(col, v);
+        ++count;
+    }
+    return count;
+}
+
+}  // namespace
+
+extern "C" {
+
+void cute_quad_release(cute_quad_lists *q)
+{
+    if (!q) return;
+    std::free(q->groupPtr);
+    std::free(q->cols);
+    std::free(q->vals);
+    std::memset(q, 0, sizeof(*q));
+}
+
+int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
+                    cute_quad_lists *out)
+{
+    if (!out || !rowPtr || (rowPtr[M] && (!cols || !vals))) return CUTE_ERR_ARG;
+    std::memset(out, 0, sizeof(*out));
+    const uint32_t P = (M + CUTE_TM - 1) / CUTE_TM;
+    out->M = M;
+    out->K = K;
+    out->numRowPanels = P;
+    out->groupPtr = cute::alloc_array<uint32_t>(uint64_t(P) + 1);
+    if (!out->groupPtr) return CUTE_ERR_NOMEM;
+
+    // sweep 1: groups per panel = ceil(longest of the four lists / 4)
+    cute::parallel_ranges(P, 64, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            uint32_t longest = 0;
+            for (uint32_t rg = 0; rg < 4; ++rg)
+                longest = std::max(longest, merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * CUTE_TM + rg * 4,
+                                                            [](uint32_t, const float *) {}));
+            out->groupPtr[q + 1] = (longest + 3) / 4;
+        }
+    });
+    uint64_t total = 0;
+    for (uint32_t q = 0; q < P; ++q) {
+        total += out->groupPtr[q + 1];
+        if (total > 0xffffffffull / 64) { cute_quad_release(out); return CUTE_ERR_SHAPE; }
+        out->groupPtr[q + 1] = uint32_t(total);
+    }
+    out->numGroups = total;
+    out->cols = cute::alloc_array<uint32_t>(total * 16);
+    out->vals = cute::alloc_array<float>(total * 64);     // calloc: absent entries are +0.0f
+    if (!out->cols || !out->vals) { cute_quad_release(out); return CUTE_ERR_NOMEM; }
+
+    // sweep 2: fill.  Steps past the end of a list repeat the list's last column (a B row the
+    // kernel has just read) with zero values; an empty list points at column 0.
+    cute::parallel_ranges(P, 64, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            const uint64_t g0 = out->groupPtr[q];
+            const uint32_t steps = (out->groupPtr[q + 1] - out->groupPtr[q]) * 4;
+            for (uint32_t rg = 0; rg < 4; ++rg) {
+                uint32_t s = 0, last = 0;
+                merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * CUTE_TM + rg * 4, [&](uint32_t col, const float *v) {
+                    const uint64_t g = g0 + s / 4;
+                    const uint32_t pair = 4 * (s % 4) + rg;
+                    out->cols[g * 16 + pair] = col;
+                    std::memcpy(out->vals + g * 64 + 4 * pair, v, 4 * sizeof(float));
+                    last = col;
+                    ++s;
+                });
+                for (; s < steps; ++s) out->cols[(g0 + s / 4) * 16 + 4 * (s % 4) + rg] = last;
+            }
+        }
+    });
+    return CUTE_OK;
+}
+
+}  // extern "C"

@@ -14,6 +14,7 @@
 namespace cute_dev {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <int VEC> struct Vec;
@@ -27,10 +28,7 @@ template <int VEC> __device__ __forceinline__ void vec_set(typename Vec<VEC>::ty
 template <> __device__ __forceinline__ void vec_set<1>(float &v, int, float x) { v = x; }
 
 constexpr int kWaveSize = 64;
-#ifndef CUTE_WPG
-#define CUTE_WPG 4
-#endif
-constexpr int kWavesPerGroup = CUTE_WPG;
+constexpr int kWavesPerGroup = 4;
 constexpr int kHdrWords = 32;
 constexpr int kNumXcd = 8;
 
@@ -104,11 +102,7 @@ __device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x
         for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-#ifdef CUTE_EXPERIMENT_NO_MFMA   // timing experiment only: keeps every load alive, drops the matrix work
-                acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
-#else
                 acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
-#endif
     }
 }
 
@@ -123,24 +117,24 @@ struct BrickItem {
     bool valid;
 };
 
+// The launch is a 2-D grid: x walks the chunks (kWavesPerGroup per work-group, remapped so that
+// each XCD owns a contiguous range), y is the slab.  gridDim.x is a multiple of the XCD count,
+// so the slabs of one chunk run on the same XCD and share its B rows in that L2.
 template <int VEC, int NG>
 __device__ __forceinline__ BrickItem brick_item(const uint4 *__restrict__ chunks, uint32_t num_chunks,
-                                                uint32_t num_slabs, uint32_t groups_per_xcd, uint32_t lane)
+                                                uint32_t groups_per_xcd, uint32_t lane)
 {
     BrickItem it;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t group = xcd_contiguous_id(blockIdx.x, groups_per_xcd);
-    const uint64_t item = uint64_t(group) * kWavesPerGroup + wave;
-    it.valid = item < uint64_t(num_chunks) * num_slabs;
+    const uint32_t chunk = xcd_contiguous_id(blockIdx.x, groups_per_xcd) * kWavesPerGroup + wave;
+    it.valid = chunk < num_chunks;
     if (!it.valid) return it;
-    const uint32_t chunk = uint32_t(item / num_slabs);
-    const uint32_t slab = uint32_t(item % num_slabs);
     const uint4 ck = chunks[chunk];
     it.start = __builtin_amdgcn_readfirstlane(ck.x);
     it.end = __builtin_amdgcn_readfirstlane(ck.y);
     it.panel = __builtin_amdgcn_readfirstlane(ck.z);
     it.atomic = __builtin_amdgcn_readfirstlane(ck.w);
-    it.col0 = slab * (16u * VEC * NG) + (lane & 15u) * VEC;
+    it.col0 = blockIdx.y * (16u * VEC * NG) + (lane & 15u) * VEC;
     return it;
 }
 
@@ -175,12 +169,12 @@ __device__ __forceinline__ void brick_store(const BrickItem &it, const f32x4 (&a
 // few wavefronts fit per SIMD anyway.
 template <int VEC, int NG, bool FULL>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd,
     const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
     float *__restrict__ C, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, num_slabs, groups_per_xcd, lane);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane);
     if (!it.valid) return;
     const uint32_t end = it.end, col0 = it.col0;
 
@@ -245,61 +239,104 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
 }
 
-// One brick's loads (A value at the lane's rank, B row segment(s)) -- the unit of the rolling
-// pipeline below.
+// One brick's loads -- the unit of the rolling pipeline below -- written for a SIMD whose
+// matrix and vector instructions share one issue stream (on gfx950 an fp32 MFMA of one
+// wavefront and the vector ALU work of another do not overlap), so every vector instruction
+// saved is time saved:
+//   * the A value is fetched already masked: lanes whose bitmap bit is clear read the zero
+//     stored behind the values (the bitmap itself, a scalar register pair, is the select mask);
+//   * the brick's value offset rides in the addend of the lane-rank count;
+//   * both addresses are 32-bit byte offsets from a scalar base (the planner checks that B and
+//     the value array are smaller than 4 GiB and that column * row pitch fits 24 x 24 bits).
+struct BrickOperands {
+    float a;
+    f32x4 b;
+};
+
+struct LeanHeader {           // like BlockHeader, plus nothing: kept separate so the scalar parts stay scalar
+    uint64_t bitmap[4];
+    uint32_t voff[4];
+    u32x4 cols;
+};
+
+__device__ __forceinline__ LeanHeader load_lean_header(const uint32_t *__restrict__ hdr, uint32_t blk, uint32_t lane)
+{
+    const uint32_t *h = hdr + size_t(blk) * kHdrWords;
+    LeanHeader r;
+    r.cols = *reinterpret_cast<const u32x4 *>(h + (lane >> 4) * 4u);
+    const uint64_t *bm = reinterpret_cast<const uint64_t *>(h + 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.bitmap[j] = bm[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.voff[j] = h[24 + j];
+    return r;
+}
+
 template <int VEC, int NG, bool FULL>
-__device__ __forceinline__ void load_brick(BlockOperands<VEC, NG> &o, int j, const BlockHeader &hd,
-                                           const float *__restrict__ vals, const float *__restrict__ B, uint32_t N,
-                                           uint32_t col0)
+__device__ __forceinline__ void load_brick_lean(typename Vec<VEC>::type (&b_out)[NG], float &a_out, int j,
+                                                const LeanHeader &hd, const float *__restrict__ vals,
+                                                uint32_t zero_index, const float *__restrict__ B, uint32_t row_pitch,
+                                                uint32_t col_off, uint32_t col0, uint32_t N)
 {
     typedef typename Vec<VEC>::type V;
-    const uint32_t cols[4] = {hd.cols.x, hd.cols.y, hd.cols.z, hd.cols.w};
     const uint64_t bm = hd.bitmap[j];
-    const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
-    o.a[j] = vals[hd.voff[j] + below];
-    o.bitmap[j] = bm;
-    const float *brow = B + size_t(cols[j]) * N + col0;
+    const uint32_t rank = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), hd.voff[j]));
+    const uint32_t aoff = (__builtin_amdgcn_inverse_ballot_w64(bm) ? rank : zero_index) * 4u;
+    a_out = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(vals) + aoff);
+    const uint32_t boff = __umul24(hd.cols[j], row_pitch) + col_off;
+    const char *brow = reinterpret_cast<const char *>(B) + boff;
 #pragma unroll
     for (int ng = 0; ng < NG; ++ng) {
-        if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + ng * 16 * VEC);
-        else o.b[j][ng] = V(0.0f);
+        if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) b_out[ng] = *reinterpret_cast<const V *>(brow + ng * 64 * VEC);
+        else b_out[ng] = V(0.0f);
     }
 }
 
-template <int VEC, int NG, bool SKIP_EMPTY>
-__device__ __forceinline__ void mfma_brick(const BlockOperands<VEC, NG> &o, int j, f32x4 (&acc)[NG][VEC], uint32_t lane)
+// C tile of one item, addressed like the loads: 32-bit byte offsets from a scalar base.
+template <int VEC, int NG, bool FULL>
+__device__ __forceinline__ void brick_store_lean(const BrickItem &it, const f32x4 (&acc)[NG][VEC], float *__restrict__ C,
+                                                 uint32_t N, uint32_t lane)
 {
-    if (SKIP_EMPTY && o.bitmap[j] == 0) return;     // wave-uniform: a brick made of padding columns only
-    const float a = ((o.bitmap[j] >> lane) & 1ull) ? o.a[j] : 0.0f;
+    typedef typename Vec<VEC>::type V;
+    const uint32_t row0 = it.panel * 16u + (lane >> 4) * 4u;
 #pragma unroll
-    for (int ng = 0; ng < NG; ++ng)
+    for (int ng = 0; ng < NG; ++ng) {
+        const uint32_t c = it.col0 + uint32_t(ng) * 16u * VEC;
+        if (!FULL && c >= N) continue;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v)
-#if defined(CUTE_EXPERIMENT_NO_MFMA)
-            acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
-#elif defined(CUTE_EXP_MFMA_BRICKS)
-            if (j < CUTE_EXP_MFMA_BRICKS) acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
-            else acc[ng][v][0] += a * vec_get<VEC>(o.b[j][ng], v);
-#else
-            acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vec_get<VEC>(o.b[j][ng], v), acc[ng][v], 0, 0, 0);
-#endif
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t off = __umul24(row0 + r, N * 4u) + c * 4u;
+            float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
+            if (it.atomic) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
+            } else {
+                V out;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
+                *reinterpret_cast<V *>(dst) = out;
+            }
+        }
+    }
 }
 
 // Variant "rolling": ONE operand set per wavefront, refilled brick by brick -- as soon as the
 // MFMAs of brick j of block i are issued, the loads of brick j of block i+1 go out into the
 // same registers.  Loads are therefore always in flight behind the MFMAs, and the register
-// budget (one operand set, one accumulator set) lets eight wavefronts share a SIMD, so a
-// launch of short panels is resident as a whole.  Padding-only bricks skip their MFMAs.
+// budget is small enough that a launch of short panels is resident as a whole.  Padding-only
+// bricks skip their MFMAs.  NG = 2 lets one wavefront cover two column groups, which halves the
+// header traffic and shares the A-side index arithmetic between them.
 template <int VEC, int NG, bool FULL>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_rolling(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t num_slabs, uint32_t groups_per_xcd,
-    const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
-    float *__restrict__ C, uint32_t N)
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_f32_rolling(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr,
+    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
+    typedef typename Vec<VEC>::type V;
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, num_slabs, groups_per_xcd, lane);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane);
     if (!it.valid) return;
-    const uint32_t end = it.end, col0 = it.col0;
+    const uint32_t end = it.end;
+    const uint32_t row_pitch = N * 4u, col_off = it.col0 * 4u;
 
     f32x4 acc[NG][VEC];
 #pragma unroll
@@ -309,279 +346,184 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_brick_f32_r
 
     uint32_t blk = it.start;
     if (blk < end) {
-        BlockOperands<VEC, NG> op;
-        BlockHeader h1, h2;
+        V b[4][NG];
+        float a[4];
+        uint64_t bitmap[4];
+        LeanHeader h1, h2;
         {
-            const BlockHeader h0 = load_header(hdr, blk, lane);
-            h1 = load_header(hdr, min(blk + 1, end - 1), lane);
+            const LeanHeader h0 = load_lean_header(hdr, blk, lane);
+            h1 = load_lean_header(hdr, min(blk + 1, end - 1), lane);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) load_brick<VEC, NG, FULL>(op, j, h0, vals, B, N, col0);
+            for (int j = 0; j < 4; ++j) {
+                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+                bitmap[j] = h0.bitmap[j];
+            }
         }
         // One basic block per iteration and a scheduling fence after every group, so the order
         // "MFMAs of brick j, then the loads that refill brick j" survives instruction scheduling.
         // Only the last block of a panel can hold padding-only bricks; it is peeled below.
-        for (; blk + 1 < end; ++blk) {       // op holds block blk, h1 the header line of blk+1
-            h2 = load_header(hdr, min(blk + 2, end - 1), lane);
+        for (; blk + 1 < end; ++blk) {       // a/b hold block blk, h1 the header line of blk+1
+            h2 = load_lean_header(hdr, min(blk + 2, end - 1), lane);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                mfma_brick<VEC, NG, false>(op, j, acc, lane);
+#pragma unroll
+                for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v)
+                        acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], vec_get<VEC>(b[j][ng], v), acc[ng][v], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                load_brick<VEC, NG, FULL>(op, j, h1, vals, B, N, col0);
+                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+                bitmap[j] = h1.bitmap[j];
                 __builtin_amdgcn_sched_barrier(0);
             }
             h1 = h2;
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) mfma_brick<VEC, NG, true>(op, j, acc, lane);
-    }
-    brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
-}
-
-// Variant "persistent": the launch holds a fixed number of wavefronts (a few per SIMD); each
-// walks a contiguous run of work items, items[i] = {first block, end block, panel,
-// atomic | slab << 1}.  Nothing but the first header fetch of a wavefront is exposed: header
-// lines run two blocks ahead ACROSS item boundaries (the descriptors of the next two items
-// are kept in scalar registers), and the store of one item overlaps the loads of the next.
-// wave_items[w] .. wave_items[w+1] is the run of logical wavefront w; logical ids are laid
-// out so that each XCD owns one contiguous range of items.
-template <int VEC, int NG, bool FULL>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32_persistent(
-    const uint4 *__restrict__ items, const uint32_t *__restrict__ wave_items, uint32_t waves_per_xcd,
-    const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
-    float *__restrict__ C, uint32_t N)
-{
-    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t logical = (blockIdx.x % kNumXcd) * waves_per_xcd + (blockIdx.x / kNumXcd) * kWavesPerGroup + wave;
-    const uint32_t ib = wave_items[logical], ie = wave_items[logical + 1];
-    if (ib >= ie) return;
-
-    struct Item { uint32_t start, end, panel, flags; };
-    auto fetch = [&](uint32_t i) {
-        const uint4 q = items[min(i, ie - 1)];          // clamped: past the run the last item repeats
-        Item r;
-        r.start = __builtin_amdgcn_readfirstlane(q.x);
-        r.end = __builtin_amdgcn_readfirstlane(q.y);
-        r.panel = __builtin_amdgcn_readfirstlane(q.z);
-        r.flags = __builtin_amdgcn_readfirstlane(q.w);
-        return r;
-    };
-    Item cur = fetch(ib), nx1 = fetch(ib + 1), nx2 = fetch(ib + 2);
-    // block id `ahead` (1 or 2) steps after block `blk` of the current item, in stream order
-    auto lookahead = [&](uint32_t blk, uint32_t ahead) {
-        if (blk + ahead < cur.end) return blk + ahead;
-        const uint32_t over = blk + ahead - cur.end, len1 = nx1.end - nx1.start;
-        return over < len1 ? nx1.start + over : nx2.start + (over - len1);
-    };
-
-    f32x4 acc[NG][VEC];
-#pragma unroll
-    for (int ng = 0; ng < NG; ++ng)
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
-
-    // Rolling refill across item boundaries: `op` holds the current block of the stream, h1 the
-    // header line of the next block of the stream (possibly the first block of the next item,
-    // whose slab -- hence B column offset -- may differ), h2 the one after that.
-    auto col0_of = [&](const Item &q) { return (q.flags >> 1) * (16u * VEC * NG) + (lane & 15u) * VEC; };
-    BlockOperands<VEC, NG> op;
-    uint32_t item = ib, blk = cur.start;
-    BlockHeader h1, h2;
-    {
-        const BlockHeader h0 = load_header(hdr, blk, lane);
-        h1 = load_header(hdr, lookahead(blk, 1), lane);
-        const uint32_t c0 = col0_of(cur);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) load_brick<VEC, NG, FULL>(op, j, h0, vals, B, N, c0);
-    }
-    while (true) {
-        const bool last_of_item = blk + 1 == cur.end;
-        const uint32_t col0_next = last_of_item ? col0_of(nx1) : col0_of(cur);
-        const uint32_t blk_next = lookahead(blk, 1);
-        h2 = load_header(hdr, lookahead(blk, 2), lane);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
         for (int j = 0; j < 4; ++j) {
-            mfma_brick<VEC, NG, false>(op, j, acc, lane);
-            __builtin_amdgcn_sched_barrier(0);
-            load_brick<VEC, NG, FULL>(op, j, h1, vals, B, N, col0_next);   // past the run: a harmless re-read
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        h1 = h2;
-        if (last_of_item) {
-            BrickItem done;
-            done.panel = cur.panel;
-            done.atomic = cur.flags & 1u;
-            done.col0 = col0_of(cur);
-            brick_store<VEC, NG, FULL>(done, acc, C, N, lane);
+            if (bitmap[j] == 0) continue;     // wave-uniform: a brick made of padding columns only
 #pragma unroll
             for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
-            if (++item == ie) break;
-            cur = nx1;
-            nx1 = nx2;
-            nx2 = fetch(item + 2);
+                for (int v = 0; v < VEC; ++v)
+                    acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], vec_get<VEC>(b[j][ng], v), acc[ng][v], 0, 0, 0);
         }
-        blk = blk_next;
     }
+    brick_store_lean<VEC, NG, FULL>(it, acc, C, N, lane);
 }
 
 // ---------------------------------------------------------------------------------------
-// Variant "stream": persistent wavefronts, each with a ring of DEPTH operand sets in registers.
+// Quad kernel: v_mfma_f32_4x4x1_16B_f32 over the quad lists (see cute_quad_lists).
 //
-// In the variants above every wavefront of a launch asks for its first operands at the same
-// moment and writes its C tile at the same moment, so the matrix pipes idle while the first
-// loads and the last stores are served.  Here a few wavefronts per SIMD each walk a long run
-// of blocks: the loads of block t+DEPTH are issued as soon as the MFMAs of block t have been
-// issued, C tiles are written (without waiting for them) while the following blocks are already
-// in flight, and the matrix pipe starts as soon as the first block of a run has landed.
+// With cbsz = 4 the instruction takes the four A values of lanes 4p..4p+3 (abid = p), and
+// multiplies them into all 64 B lanes: D[i][lane] += A[4p+i] * B[lane].  One instruction is
+// therefore "one column of one 4-row group times 64 output columns" -- 8 cycles of the SIMD
+// instead of the 36 a 16x16x4 tile costs, and a panel only pays for the (row group, column)
+// pairs that hold a nonzero.
 //
-// The host flattens the work into one stream of blocks per wavefront:
-//   step_blk[t]   block id
-//   step_meta[t]  low word: row panel; high word: flags
-//                 flags bit0 last step of its item (store C afterwards),
-//                       bit1 combine through atomics,
-//                       bit2 padding step (items are padded to a whole number of ring turns),
-//                       bits 8.. slab index (64 columns per slab)
-// wave_steps[w] .. wave_steps[w+1] is the run of logical wavefront w (XCD-contiguous ids); runs
-// end on item boundaries.  Both step arrays are padded by DEPTH+2 repeats of the last step, so
-// look-ahead never leaves them.
+// Lane L owns output column slab*64 + L of all 16 rows: acc[rg][i] is row 4*rg+i.  A group's
+// 64 values are one coalesced dword per lane and ARE the A register (lane 4p+i = pair p, row i);
+// its 16 columns are wave-uniform (scalar registers); its 16 B operands are one dword per lane
+// each, a contiguous 256-byte piece of a B row.  Two operand sets roll: as soon as the MFMA of
+// pair p is issued, B operand p of the group after next is requested into the same register.
 //
-// Header lines are wave-uniform and are fetched with scalar loads only; every block issues
-// exactly eight vector loads (4 A, 4 B), also past the end of a run (there the B part is pointed
-// at the zero pad behind the values), so the number of loads in flight behind any operand set
-// is a compile-time constant and the waits never drain the ring.
+// chunks[i] = {first group, end group, row panel, atomic}; launch: x walks the chunks, y the slabs.
+// Addresses are 32-bit byte offsets from scalar bases; the planner checks the sizes.
 // ---------------------------------------------------------------------------------------
-struct ScalarHeader {        // a whole header line in scalar registers
-    uint32_t cols[16];
-    uint64_t bitmap[4];
-    uint32_t voff[4];
-};
-
-__device__ __forceinline__ ScalarHeader load_scalar_header(const uint32_t *__restrict__ hdr, uint32_t blk)
+template <int P>
+__device__ __forceinline__ void quad_mfma(float a, float b, f32x4 (&acc)[4])
 {
-    const uint32_t *h = hdr + size_t(blk) * kHdrWords;
-    ScalarHeader r;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) r.cols[i] = h[i];
-    const uint64_t *bm = reinterpret_cast<const uint64_t *>(h + 16);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) r.bitmap[j] = bm[j];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) r.voff[j] = h[24 + j];
-    return r;
+    acc[P & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, acc[P & 3], 4, P, 0);
 }
 
-struct StreamOperands {      // one block: masked A values and B row segments of its four bricks
-    float a[4];
-    f32x4 b[4];
-};
-
-// keep == 0 (padding step, or a step past the end of the run) turns every A value into the stored zero.
-__device__ __forceinline__ void stream_issue(StreamOperands &o, const ScalarHeader &h, const float *__restrict__ vals,
-                                             uint32_t keep, uint32_t zero_index, const float *__restrict__ B, uint32_t N,
-                                             uint32_t col, uint32_t lane)
+__device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32_t col, uint32_t row_pitch, uint32_t col_off)
 {
-    const uint32_t g = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        // column of lane group g in brick j: header word g*4 + j
-        const uint32_t c01 = g == 0 ? h.cols[j] : h.cols[4 + j];
-        const uint32_t c23 = g == 2 ? h.cols[8 + j] : h.cols[12 + j];
-        const uint32_t colj = g < 2 ? c01 : c23;
-        const uint64_t bm = h.bitmap[j] & (uint64_t(keep) | (uint64_t(keep) << 32));
-        const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
-        // lanes whose bit is clear read a stored zero, so the register holds the masked A operand
-        const uint32_t aidx = ((bm >> lane) & 1ull) ? h.voff[j] + below : zero_index;
-        o.a[j] = vals[aidx];
-        o.b[j] = *reinterpret_cast<const f32x4 *>(B + size_t(colj) * N + col);
-    }
+    return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(B) + (__umul24(col, row_pitch) + col_off));
 }
 
-template <int DEPTH, bool FULL>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32_stream(
-    const uint32_t *__restrict__ step_blk, const uint64_t *__restrict__ step_meta, const uint32_t *__restrict__ wave_steps,
-    uint32_t waves_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ vals, uint32_t zero_index,
-    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+template <bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
+    const float *__restrict__ qvals, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
-    static_assert(DEPTH >= 2 && DEPTH <= 6, "ring depth");
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t logical = (blockIdx.x % kNumXcd) * waves_per_xcd + (blockIdx.x / kNumXcd) * kWavesPerGroup + wave;
-    const uint32_t t0 = wave_steps[logical], t1 = wave_steps[logical + 1];
-    if (t0 >= t1) return;
-    const uint32_t lane_col = (lane & 15u) * 4u;
-    auto column_of = [&](uint32_t flags) {
-        const uint32_t c = (flags >> 8) * 64u + lane_col;
-        return FULL ? c : min(c, N - 4u);          // ragged tail: re-read the last full vector, masked at the store
-    };
-    const float *zeros = vals + zero_index;
+    const uint32_t chunk = xcd_contiguous_id(blockIdx.x, groups_per_xcd) * kWavesPerGroup + wave;
+    if (chunk >= num_chunks) return;
+    const uint4 ck = chunks[chunk];
+    const uint32_t g_end = __builtin_amdgcn_readfirstlane(ck.y);
+    const uint32_t panel = __builtin_amdgcn_readfirstlane(ck.z);
+    const uint32_t atomic = __builtin_amdgcn_readfirstlane(ck.w);
+    uint32_t g = __builtin_amdgcn_readfirstlane(ck.x);
 
-    StreamOperands ring[DEPTH];
-    // prologue: fill the ring
-#pragma unroll
-    for (int i = 0; i < DEPTH; ++i) {
-        const ScalarHeader h = load_scalar_header(hdr, step_blk[t0 + i]);
-        const uint32_t f = uint32_t(step_meta[t0 + i] >> 32);
-        const bool live = !(f & 4u);              // a run holds at least one whole item, i.e. DEPTH steps
-        stream_issue(ring[i], h, vals, live ? 0xffffffffu : 0u, zero_index, live ? B : zeros, live ? N : 0u,
-                     live ? column_of(f) : lane_col, lane);
-    }
-    // scalar look-ahead: header of step t+DEPTH (used at the end of step t), block id of t+DEPTH+1
-    ScalarHeader h_issue = load_scalar_header(hdr, step_blk[t0 + DEPTH]);
-    uint32_t blk_ahead = step_blk[t0 + DEPTH + 1];
-    uint32_t flags_issue = uint32_t(step_meta[t0 + DEPTH] >> 32);
+    const uint32_t n = blockIdx.y * kWaveSize + lane;
+    const bool live = FULL || n < N;
+    const uint32_t row_pitch = N * 4u;
+    const uint32_t col_off = (live ? n : N - 1u) * 4u;      // dead lanes re-read the last column and store nothing
 
-    uint32_t t = t0;
-    do {   // one item: a whole number of ring turns that ends with a C tile
-        f32x4 acc[4];
+    f32x4 acc[4];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[v] = f32x4(0.0f);
-        uint64_t meta;
-        do {   // one ring turn
+    for (int rg = 0; rg < 4; ++rg) acc[rg] = f32x4(0.0f);
+
+    if (g < g_end) {
+        // Two operand sets, so every B operand is requested two groups before its MFMA: set 0 holds
+        // group g, set 1 group g+1 (or a harmless re-read of the last group when there is none).
+        float b0[16], b1[16], a0, a1;
+        uint32_t ca[16], cb[16];       // column lists of the groups being requested (scalar registers)
+        const uint32_t last = g_end - 1u;
+        auto fetch_cols = [&](uint32_t (&c)[16], uint32_t grp) {
+            const uint32_t *src = qcols + size_t(min(grp, last)) * 16u;
 #pragma unroll
-            for (int s = 0; s < DEPTH; ++s) {
-                StreamOperands &o = ring[s];
+            for (int p = 0; p < 16; ++p) c[p] = src[p];
+        };
+        auto fetch_a = [&](uint32_t grp) { return qvals[size_t(min(grp, last)) * 64u + lane]; };
+        fetch_cols(ca, g);
+        fetch_cols(cb, g + 1);
+        a0 = fetch_a(g);
+        a1 = fetch_a(g + 1);
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+        for (int p = 0; p < 16; ++p) b0[p] = quad_load_b(B, ca[p], row_pitch, col_off);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v)
-                        acc[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[j], o.b[j][v], acc[v], 0, 0, 0);
-                // refill the set just consumed with block t+s+DEPTH, then advance the scalar look-ahead
-                {
-                    const bool live = !(flags_issue & 4u) && t + s + DEPTH < t1;
-                    stream_issue(o, h_issue, vals, live ? 0xffffffffu : 0u, zero_index, live ? B : zeros, live ? N : 0u,
-                                 live ? column_of(flags_issue) : lane_col, lane);
-                }
-                h_issue = load_scalar_header(hdr, blk_ahead);
-                flags_issue = uint32_t(step_meta[t + s + DEPTH + 1] >> 32);
-                blk_ahead = step_blk[t + s + DEPTH + 2];
-            }
-            meta = step_meta[t + DEPTH - 1];
-            t += DEPTH;
-        } while (!(uint32_t(meta >> 32) & 1u));
-        // end of the item: write its C tile; the stores are not waited for
-        const uint32_t flags = uint32_t(meta >> 32);
-        const uint32_t c = (flags >> 8) * 64u + lane_col;
-        if (FULL || c < N) {
-            const uint32_t row0 = uint32_t(meta) * 16u + (lane >> 4) * 4u;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float *dst = C + size_t(row0 + r) * N + c;
-                if (flags & 2u) {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) unsafeAtomicAdd(dst + v, acc[v][r]);
-                } else {
-                    f32x4 out;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) out[v] = acc[v][r];
-                    *reinterpret_cast<f32x4 *>(dst) = out;
-                }
-            }
+        for (int p = 0; p < 16; ++p) b1[p] = quad_load_b(B, cb[p], row_pitch, col_off);
+#define CUTE_QUAD_ROLL(P, A, BSET, COLS)                          \
+    quad_mfma<P>(A, BSET[P], acc);                                \
+    __builtin_amdgcn_sched_barrier(0);                            \
+    BSET[P] = quad_load_b(B, COLS[P], row_pitch, col_off);        \
+    __builtin_amdgcn_sched_barrier(0);
+#define CUTE_QUAD_ROLL_REST(A, BSET, COLS)                                                                 \
+    CUTE_QUAD_ROLL(1, A, BSET, COLS) CUTE_QUAD_ROLL(2, A, BSET, COLS)                                      \
+    CUTE_QUAD_ROLL(3, A, BSET, COLS) CUTE_QUAD_ROLL(4, A, BSET, COLS) CUTE_QUAD_ROLL(5, A, BSET, COLS)    \
+    CUTE_QUAD_ROLL(6, A, BSET, COLS) CUTE_QUAD_ROLL(7, A, BSET, COLS) CUTE_QUAD_ROLL(8, A, BSET, COLS)    \
+    CUTE_QUAD_ROLL(9, A, BSET, COLS) CUTE_QUAD_ROLL(10, A, BSET, COLS) CUTE_QUAD_ROLL(11, A, BSET, COLS)  \
+    CUTE_QUAD_ROLL(12, A, BSET, COLS) CUTE_QUAD_ROLL(13, A, BSET, COLS) CUTE_QUAD_ROLL(14, A, BSET, COLS) \
+    CUTE_QUAD_ROLL(15, A, BSET, COLS)
+#define CUTE_QUAD_MFMA16(A, BSET)                                                                          \
+    quad_mfma<0>(A, BSET[0], acc);   quad_mfma<1>(A, BSET[1], acc);   quad_mfma<2>(A, BSET[2], acc);       \
+    quad_mfma<3>(A, BSET[3], acc);   quad_mfma<4>(A, BSET[4], acc);   quad_mfma<5>(A, BSET[5], acc);       \
+    quad_mfma<6>(A, BSET[6], acc);   quad_mfma<7>(A, BSET[7], acc);   quad_mfma<8>(A, BSET[8], acc);       \
+    quad_mfma<9>(A, BSET[9], acc);   quad_mfma<10>(A, BSET[10], acc); quad_mfma<11>(A, BSET[11], acc);     \
+    quad_mfma<12>(A, BSET[12], acc); quad_mfma<13>(A, BSET[13], acc); quad_mfma<14>(A, BSET[14], acc);     \
+    quad_mfma<15>(A, BSET[15], acc);
+        fetch_cols(ca, g + 2);
+        while (g + 2 < g_end) {              // groups g, g+1 and g+2 exist
+            // group g from set 0; set 0 is refilled with group g+2.  The other column list is
+            // asked for right after this one's first use (where it is waited for), so that wait
+            // never covers a fetch just issued; it is first used 15 pairs later.
+            const float a0n = fetch_a(g + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            CUTE_QUAD_ROLL(0, a0, b0, ca)
+            fetch_cols(cb, g + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            CUTE_QUAD_ROLL_REST(a0, b0, ca)
+            a0 = a0n;
+            // group g+1 from set 1; set 1 is refilled with group g+3 (clamped to the last one)
+            const float a1n = fetch_a(g + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            CUTE_QUAD_ROLL(0, a1, b1, cb)
+            fetch_cols(ca, g + 4);
+            __builtin_amdgcn_sched_barrier(0);
+            CUTE_QUAD_ROLL_REST(a1, b1, cb)
+            a1 = a1n;
+            g += 2;
         }
-    } while (t < t1);
+        CUTE_QUAD_MFMA16(a0, b0)
+        if (g + 1 < g_end) { CUTE_QUAD_MFMA16(a1, b1) }
+#undef CUTE_QUAD_ROLL
+#undef CUTE_QUAD_ROLL_REST
+#undef CUTE_QUAD_MFMA16
+    }
+    if (live) {
+        uint32_t off = __umul24(panel * 16u, row_pitch) + n * 4u;
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
+                if (atomic) unsafeAtomicAdd(dst, acc[rg][i]);
+                else *dst = acc[rg][i];
+                off += row_pitch;
+            }
+    }
 }
 
 // Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).

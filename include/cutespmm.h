@@ -121,6 +121,29 @@ int cute_hrpb_untile(const cute_hrpb_tiled *t, cute_hrpb_host *out);
 void cute_hrpb_tiled_release(cute_hrpb_tiled *t);
 
 /* ------------------------------------------------------------------------------------
+ * host: quad lists, the layout of the 4x4x1 MFMA kernel.  No counterpart in the reference
+ * (its kernel consumes the brick stream directly, kernel.cu:88-125); derived from the same CSR
+ * input as cute_hrpb_build.  Each 4-row group of a panel has its own sorted list of active
+ * columns; the four lists of a panel advance in lockstep, padded to the longest.  One group
+ * of the layout is 16 (row group, column) pairs = 4 steps x 4 row groups:
+ *   cols[g*16 + 4*s + rg]            column of row group rg at step s of group g
+ *   vals[g*64 + 4*(4*s + rg) + i]    value of row 4*rg+i of the panel in that column, else 0
+ * groupPtr[q] .. groupPtr[q+1] are the groups of row panel q.  Padding steps repeat the last
+ * column of their list (column 0 for an empty list) with zero values.
+ * ---------------------------------------------------------------------------------- */
+typedef struct cute_quad_lists {
+    uint32_t M, K, numRowPanels;
+    uint64_t numGroups;
+    uint32_t *groupPtr;        /* [numRowPanels+1]                                         */
+    uint32_t *cols;            /* [numGroups*16]                                           */
+    float *vals;               /* [numGroups*64]                                           */
+} cute_quad_lists;
+
+int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
+                    cute_quad_lists *out);
+void cute_quad_release(cute_quad_lists *q);
+
+/* ------------------------------------------------------------------------------------
  * host: launch partition.            Replaces SPMM_TC::partition (spmm.cu:776-812).
  * Same arithmetic; the machine enters through `slots` (work items resident on the whole
  * device; num_sms*num_thread_blocks at spmm.cu:778-779) and `nbN` (work items along N).
@@ -239,13 +262,13 @@ uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d); /* device bytes held */
  * (spmm.cu:276-822) and SPMM_TC::run (spmm.cu:823-839).
  * ---------------------------------------------------------------------------------- */
 typedef enum cute_path {
-    CUTE_PATH_AUTO = 0,        /* per-panel choice between brick and row kernels          */
-    CUTE_PATH_BRICK = 1,       /* every panel through the MFMA brick kernel               */
+    CUTE_PATH_AUTO = 0,        /* per-panel choice between the MFMA and row kernels       */
+    CUTE_PATH_BRICK = 1,       /* every panel through the MFMA kernel (see mfma_shape)    */
     CUTE_PATH_ROWS = 2         /* every panel through the wavefront-per-row kernel        */
 } cute_path;
 
 typedef enum cute_precision {
-    CUTE_PREC_FP32 = 0,        /* v_mfma_f32_16x16x4_f32, fp32 operands                   */
+    CUTE_PREC_FP32 = 0,        /* fp32 MFMA (4x4x1 or 16x16x4), fp32 operands             */
     CUTE_PREC_BF16X3 = 1       /* bf16 hi/lo split, three bf16 MFMA products              */
 } cute_precision;
 
@@ -256,8 +279,8 @@ typedef struct cute_tunables {
     uint32_t slots;            /* resident work items assumed by the partition; 0: derive from device */
     uint32_t max_chunk_blocks; /* upper bound on blocks per work item; 0: none            */
     uint32_t brick_groups;     /* 16-lane column groups per lane in the brick kernel (1 or 2); 0: default */
-    uint32_t pipeline;         /* brick kernel variant: 1 resident, 2 pipelined, 3 persistent; 0: default          */
-    uint32_t waves_per_cu;     /* persistent variant: wavefronts launched per CU; 0: default                      */
+    uint32_t pipeline;         /* brick kernel variant: 1 rolling, 2 pipelined; 0: default (rolling)             */
+    uint32_t mfma_shape;       /* MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists; 0: default (quad lists)     */
     uint32_t max_row_nnz;      /* AUTO: panels holding a row longer than this stay on the brick kernel; 0: default  */
     uint32_t reserved[3];
 } cute_tunables;

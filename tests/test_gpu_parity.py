@@ -37,8 +37,13 @@ def _run(cs, torch, h, B, **kw):
 
 
 def _paths(cs):
-    return [("brick", dict(path=cs.PATH_BRICK)), ("brick_g1", dict(path=cs.PATH_BRICK, brick_groups=1)),
-            ("rows", dict(path=cs.PATH_ROWS)), ("auto", dict())]
+    mfma = dict(path=cs.PATH_BRICK)
+    return [("quad", dict(mfma, mfma_shape=2)),
+            ("brick_rolling", dict(mfma, mfma_shape=1, pipeline=1)),
+            ("brick_rolling_g2", dict(mfma, mfma_shape=1, pipeline=1, brick_groups=2)),
+            ("brick_pipelined", dict(mfma, mfma_shape=1, pipeline=2)),
+            ("brick_pipelined_g2", dict(mfma, mfma_shape=1, pipeline=2, brick_groups=2)),
+            ("mfma_default", mfma), ("rows", dict(path=cs.PATH_ROWS)), ("auto", dict())]
 
 
 def test_device_is_gfx950(cs, torch_cuda):
@@ -154,13 +159,14 @@ def test_split_panels_combine_through_atomics(cs, orc, torch_cuda):
     B = rng.standard_normal((K, N)).astype(np.float32)
     ref = orc.spmm_csr(rp, cl, vl, B)
     h = cs.HRPB(M, K, rp, cl, vl)
-    out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK)
-    assert plan.info["numAtomicChunks"] > 0
-    assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
-    # forcing tiny chunks everywhere, and the reference's own partition arithmetic
-    for kw in (dict(max_chunk_blocks=1), dict(max_chunk_blocks=3), dict(slots=64), dict(slots=864)):
-        out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, **kw)
-        assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, kw
+    for shape in (1, 2):
+        out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=shape)
+        assert plan.info["numAtomicChunks"] > 0
+        assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
+        # forcing tiny chunks everywhere, and the reference's own partition arithmetic
+        for kw in (dict(max_chunk_blocks=1), dict(max_chunk_blocks=3), dict(slots=64), dict(slots=864)):
+            out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=shape, **kw)
+            assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (shape, kw)
     # a second launch on the same output buffer must not accumulate on top of the first
     import torch
     dB = torch.from_numpy(B).cuda()

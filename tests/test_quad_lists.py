@@ -1,0 +1,82 @@
+"""Quad lists (the 4x4x1 MFMA kernel's layout): structure and exact content, on the CPU.
+
+The layout has no counterpart in the reference, so it is pinned by what defines it: decoding it
+must give back the CSR matrix bit for bit, each row group's columns must ascend strictly over its
+real steps, the four lists of a panel must be padded to one common length, and that length must be
+the shortest one possible (some row group really has that many distinct columns)."""
+import numpy as np
+import pytest
+
+from helpers import random_csr
+
+
+def _decode(M, K, q):
+    """(row, col) -> value for every non-padding slot, plus per-(panel, row group) real lengths."""
+    gp = q["groupPtr"].astype(np.int64)
+    entries = {}
+    for p in range(len(gp) - 1):
+        for g in range(gp[p], gp[p + 1]):
+            for pair in range(16):
+                rg, col = pair % 4, int(q["cols"][g, pair])
+                for i in range(4):
+                    v = q["vals"][g, 4 * pair + i]
+                    if v != 0:
+                        key = (16 * p + 4 * rg + i, col)
+                        assert key not in entries, "a matrix entry appears twice"
+                        entries[key] = v
+    return entries
+
+
+def _cases():
+    rng = np.random.default_rng(11)
+    yield "random", (64, 96) + random_csr(rng, 64, 96, density=0.1)
+    yield "empty_rows", (48, 64) + random_csr(rng, 48, 64, density=0.2, empty_rows=set(range(16, 32)) | {3, 40})
+    yield "dense_panel", (16, 32) + random_csr(rng, 16, 32, density=1.0)
+    yield "single", (16, 16) + random_csr(rng, 16, 16, row_nnz=lambda r: 1 if r == 5 else 0)
+    yield "all_empty", (32, 16) + random_csr(rng, 32, 16, row_nnz=0)
+    yield "long_row", (32, 4096) + random_csr(rng, 32, 4096, row_nnz=lambda r: 3000 if r == 17 else 2)
+
+
+@pytest.mark.parametrize("name,case", list(_cases()), ids=[n for n, _ in _cases()])
+def test_quad_lists_hold_exactly_the_matrix(cs, name, case):
+    M, K, rp, cl, vl = case
+    q = cs.quad_lists(M, K, rp, cl, vl)
+    gp = q["groupPtr"].astype(np.int64)
+    assert gp[0] == 0 and gp[-1] == q["numGroups"] and len(gp) == M // 16 + 1 and (np.diff(gp) >= 0).all()
+    assert q["cols"].shape == (q["numGroups"], 16) and q["vals"].shape == (q["numGroups"], 64)
+    assert (q["cols"] < K).all()
+    entries = _decode(M, K, q)
+    expect = {(r, int(cl[k])): vl[k] for r in range(M) for k in range(rp[r], rp[r + 1]) if vl[k] != 0}
+    assert entries.keys() == expect.keys()
+    assert all(np.float32(entries[k]).tobytes() == np.float32(expect[k]).tobytes() for k in expect)
+    # structure of every panel
+    for p in range(M // 16):
+        longest = 0
+        for rg in range(4):
+            rows = range(16 * p + 4 * rg, 16 * p + 4 * rg + 4)
+            want = sorted({int(c) for r in rows for c in cl[rp[r]:rp[r + 1]]})
+            longest = max(longest, len(want))
+            steps = [int(q["cols"][g, 4 * s + rg]) for g in range(gp[p], gp[p + 1]) for s in range(4)]
+            assert steps[:len(want)] == want, (name, p, rg)                       # ascending, complete
+            pad = want[-1] if want else 0
+            assert all(c == pad for c in steps[len(want):]), (name, p, rg)        # padding repeats the last column
+            for t in range(len(want), len(steps)):                                # ... with zero values
+                g, s = gp[p] + t // 4, t % 4
+                assert not q["vals"][g, 4 * (4 * s + rg):4 * (4 * s + rg) + 4].any()
+        assert gp[p + 1] - gp[p] == (longest + 3) // 4, (name, p)
+
+
+def test_quad_lists_of_the_golden_matrix(cs):
+    import os
+    from test_oracle_pins import GOLD
+    r = cs.MTX_READER(os.path.join(GOLD, "G67.mtx"))
+    q = cs.quad_lists(r.M, r.K, r.rowPtr, r.cols, r.vals)
+    assert np.count_nonzero(q["vals"]) == r.nnz
+    # a toroidal 4-neighbour grid: a 4-row group of consecutive vertices touches at most 16 columns
+    assert q["numGroups"] <= 4 * (r.M // 16)
+
+
+def test_quad_build_rejects_null_arguments(cs):
+    import ctypes as C
+    lib = cs.load_library()
+    assert lib.cute_quad_build(16, 16, None, None, None, None) == -5
