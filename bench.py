@@ -4,10 +4,11 @@
 A step is one SpMM (C = A.B) over the headline workload: the 65536-row 9-point-stencil
 matrix with a dense 65536 x 128 fp32 B, inputs resident in HBM before timing starts.
 Prints ONE JSON line: GFLOP/s = 2.nnz.N / t, the HBM roofline of the dominant kernel
-(algorithmic bytes / per-launch kernel time from HIP events on the launch stream) and
+(algorithmic bytes / average launch duration from HIP events around the timed launches) and
 the CPU oracle timed on the host cores as a reported baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu] [--detail FILE]
+                    [--path auto|mfma|rows] [--mfma-shape 0|1|2] [--pipeline 0|1|2] [--calibrate-copy]
 """
 import argparse
 import json
@@ -67,6 +68,11 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--detail", default=None, help="also time every path and the CSR kernels; write JSON here")
+    ap.add_argument("--path", choices=("auto", "mfma", "rows"), default="auto", help="kernel family (default: the planner's choice)")
+    ap.add_argument("--mfma-shape", type=int, default=0, help="1: 16x16x4 brick kernel, 2: 4x4x1 quad kernel, 0: planner's choice")
+    ap.add_argument("--pipeline", type=int, default=0, help="brick kernel variant: 1 rolling, 2 pipelined, 0: default")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run 10 plain device copies of 32 MiB and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (got --gpus %d); nothing here shards across GPUs" % args.gpus)
@@ -76,6 +82,14 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    if args.calibrate_copy:
+        src = torch.arange(8 << 20, dtype=torch.float32, device="cuda")      # 32 MiB read, 32 MiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps(dict(copy_bytes_read=src.numel() * 4, copy_bytes_written=dst.numel() * 4, copies=10)))
+        return
     cfg = cs.CONFIGS[args.config]
     A = cs.gen_config(args.config)
     N = cfg["N"]
@@ -83,29 +97,43 @@ def main():
     h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
     dB = torch.from_numpy(B).cuda()
     dC = torch.empty((A.M, N), device="cuda")
-    plan = cs.SPMM_TC(h, N)
+    plan = cs.SPMM_TC(h, N, path={"auto": cs.PATH_AUTO, "mfma": cs.PATH_BRICK, "rows": cs.PATH_ROWS}[args.path],
+                      mfma_shape=args.mfma_shape, pipeline=args.pipeline)
     stream = torch.cuda.current_stream()
 
     for _ in range(args.warmup):
         plan.run(dB, dC)
     torch.cuda.synchronize()
+    # the timed region: exactly K steps, synchronised on both sides; HIP events on the launch
+    # stream bracket the same K launches and give the average launch duration for the roofline
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record(stream)
     for _ in range(args.steps):
         plan.run(dB, dC)
+    ev1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     flops = 2.0 * A.nnz * N
     value = flops / (ms_per_step * 1e-3) / 1e9
 
-    # dominant kernel: per-launch duration from HIP events on the launch stream
-    ms = plan.time(dB, dC, warmup=5, iters=max(20, min(args.steps, 200)), stream=stream)
-    kernel_ms = float(np.mean(ms))
+    kernel_ms = ev0.elapsed_time(ev1) / args.steps
+    # the same launches one by one, each inside its own event pair (adds the cost of the bracket)
+    each = plan.time(dB, dC, warmup=5, iters=max(20, min(args.steps, 200)), stream=stream)
     abytes = algorithmic_bytes(A.M, A.K, N, A.nnz)
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    kernels = []
+    if plan.info["numAtomicChunks"]:
+        kernels.append("zero_panels")
+    if plan.info["numChunks"]:
+        kernels.append(plan.kernel_name)
+    if plan.info["numRowPanelsSparse"] or plan.info["numEmptyPanels"]:
+        kernels.append("csr_rows_batched")
     roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                    traffic=recorded_traffic(cfg["name"]), kernel="hrpb_brick_f32" if plan.info["numChunks"] else "csr_rows",
-                    kernel_ms=kernel_ms, kernel_ms_median=float(np.median(ms)), algorithmic_bytes=abytes)
+                    traffic=recorded_traffic(cfg["name"]), kernel=plan.kernel_name if plan.info["numChunks"] else "csr_rows_batched",
+                    kernels_per_step=kernels, kernel_ms=kernel_ms, kernel_ms_single_bracketed_median=float(np.median(each)),
+                    algorithmic_bytes=abytes)
 
     out = dict(metric="SpMM GFLOP/s (2*nnz*N/t) on 1 MI355X", value=value, unit="GFLOP/s", n_gpus=1,
                steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
@@ -125,8 +153,9 @@ def main():
 
     if args.detail:
         detail = dict(workload=cfg["name"], paths={}, csr={})
-        for name, kw in (("brick_groups2", dict(path=cs.PATH_BRICK, brick_groups=2)),
-                         ("brick_groups1", dict(path=cs.PATH_BRICK, brick_groups=1)),
+        for name, kw in (("quad", dict(path=cs.PATH_BRICK, mfma_shape=2)),
+                         ("brick_rolling", dict(path=cs.PATH_BRICK, mfma_shape=1, pipeline=1)),
+                         ("brick_pipelined", dict(path=cs.PATH_BRICK, mfma_shape=1, pipeline=2)),
                          ("rows", dict(path=cs.PATH_ROWS)), ("auto", dict())):
             p = cs.SPMM_TC(h, N, **kw)
             t = p.time(dB, dC, warmup=5, iters=50, stream=stream)

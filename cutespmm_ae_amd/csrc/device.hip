@@ -377,6 +377,8 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->info.slots = slots;
     p->info.precision = uint32_t(t.precision);
     p->info.path = uint32_t(t.path);
+    p->info.mfmaShape = uint32_t(p->shape);
+    p->info.pipeline = uint32_t(p->pipeline);
     *out = p;
     return CUTE_OK;
 }

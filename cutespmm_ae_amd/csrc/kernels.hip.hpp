@@ -158,7 +158,7 @@ __device__ __forceinline__ void brick_store(const BrickItem &it, const f32x4 (&a
                 V out;
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
-                *reinterpret_cast<V *>(dst) = out;
+                __builtin_nontemporal_store(out, reinterpret_cast<V *>(dst));   // C is not read again: keep it out of the L2
             }
         }
     }
@@ -314,7 +314,7 @@ __device__ __forceinline__ void brick_store_lean(const BrickItem &it, const f32x
                 V out;
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
-                *reinterpret_cast<V *>(dst) = out;
+                __builtin_nontemporal_store(out, reinterpret_cast<V *>(dst));   // C is not read again: keep it out of the L2
             }
         }
     }
@@ -520,7 +520,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
             for (int i = 0; i < 4; ++i) {
                 float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
                 if (atomic) unsafeAtomicAdd(dst, acc[rg][i]);
-                else *dst = acc[rg][i];
+                else __builtin_nontemporal_store(acc[rg][i], dst);   // C is not read again: keep it out of the L2
                 off += row_pitch;
             }
     }
@@ -622,7 +622,7 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
             for (uint32_t u = 0; u < STEP; ++u) acc += a[u] * b[u];
         }
     }
-    if (live) *reinterpret_cast<V *>(C + size_t(row) * N + c0) = acc;
+    if (live) __builtin_nontemporal_store(acc, reinterpret_cast<V *>(C + size_t(row) * N + c0));
 }
 
 // Thread per C element (inc/SPMM.cuh:898-920 restated for fp32 and a 64x4 thread tile).

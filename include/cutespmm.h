@@ -294,7 +294,9 @@ typedef struct cute_plan_info {
     uint32_t numBrickPanels, numRowPanelsSparse, numEmptyPanels;
     uint32_t slots;
     uint32_t precision, path;
-    uint32_t reserved[5];
+    uint32_t mfmaShape;        /* MFMA kernel in use: 1 16x16x4 bricks, 2 4x4x1 quad lists */
+    uint32_t pipeline;         /* brick kernel variant in use: 1 rolling, 2 pipelined     */
+    uint32_t reserved[3];
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;
