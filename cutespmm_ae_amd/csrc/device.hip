@@ -243,6 +243,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (t.precision != CUTE_PREC_FP32) return CUTE_ERR_ARG;   // the bf16x3 kernel is not built yet
     const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : 1.25f;
     const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : 48;   // measured: longer rows serialise a lane group
+    // An MFMA work item always spans 64 output columns; when N is narrower the row kernel wastes
+    // less, so the reuse a panel must offer to earn the MFMA kernel grows (measured on N = 8..32).
+    const float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
 
     cute_spmm_plan *p = new cute_spmm_plan;
     p->d = d;
@@ -259,7 +262,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             // Row kernel when a fetched B row serves hardly more than one nonzero of the panel
             // (the 16-row MFMA then buys nothing) -- unless a row is so long that one lane group
             // would serialise it: the brick kernel cuts long panels into balanced chunks.
-            rows = float(d->panelNnz[q]) < min_reuse * float(d->panelCols[q]) && d->panelMaxRow[q] <= max_row_for_rows;
+            rows = float(d->panelNnz[q]) < reuse_bar * float(d->panelCols[q]) && d->panelMaxRow[q] <= max_row_for_rows;
         }
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;
@@ -267,7 +270,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
-    p->ng = 1;   // one 16-lane column group per lane measured faster than two on every benchmark matrix
+    p->ng = (p->vec == 4 && N >= 128) ? 2 : 1;   // two column groups per lane pay off from 128 columns on (measured)
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
     if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
     // the rolling variant addresses B and the values with 32-bit byte offsets (24 x 24-bit product)
