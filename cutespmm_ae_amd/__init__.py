@@ -21,7 +21,7 @@ ABI_SYMBOLS = [
     "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
-    "cute_quad_build", "cute_quad_release",
+    "cute_quad_build", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
@@ -153,6 +153,8 @@ def load_library():
     lib.cute_quad_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.argtypes = [C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.restype = None
+    lib.cute_hrpb_save.argtypes = [C.POINTER(cute_hrpb_host), C.c_char_p]
+    lib.cute_hrpb_load.argtypes = [C.c_char_p, C.POINTER(cute_csr), C.POINTER(cute_hrpb_host)]
     lib.cute_partition.restype = C.c_int64
     lib.cute_partition.argtypes = [C.c_uint32, u32p, C.c_uint32, C.c_uint32, u32p, C.c_uint64]
     lib.cute_check_gemm_correctness.restype = C.c_float
@@ -353,6 +355,9 @@ class HRPB:
         self._dev = C.c_void_p()
         _check(load_library().cute_hrpb_build(int(M), int(K), _ptr(self.rowPtr, u32p), _ptr(self.cols, u32p),
                                               _ptr(self.vals, f32p), C.byref(self._raw)), "cute_hrpb_build")
+        self._publish()
+
+    def _publish(self):
         r = self._raw
         self.M, self.K = r.M, r.K
         self.numRowPanels, self.numBlocks, self.numWords = r.numRowPanels, r.numBlocks, r.numWords
@@ -362,6 +367,28 @@ class HRPB:
         self.activeCols = _view(r.activeCols, r.numBlocks * 16, np.uint32, self._guard)
         self.sizePtr = _view(r.sizePtr, r.numBlocks + 1, np.uint64, self._guard)
         self.blocksData = _view(r.blocksData, r.numWords, np.uint32, self._guard)
+
+    def save(self, path):
+        """Writes the CSR arrays and the canonical format to a versioned, checksummed binary file."""
+        _check(load_library().cute_hrpb_save(C.byref(self._raw), os.fsencode(path)), "cute_hrpb_save")
+
+    @classmethod
+    def load(cls, path):
+        """The object a previous ``save`` wrote, without reading or converting the matrix again."""
+        lib = load_library()
+        self = cls.__new__(cls)
+        csr = cute_csr()
+        self._raw = cute_hrpb_host()
+        self._dev = C.c_void_p()
+        _check(lib.cute_hrpb_load(os.fsencode(path), C.byref(csr), C.byref(self._raw)), "cute_hrpb_load")
+        # the CSR arrays move into numpy-owned memory, which the format object then borrows
+        self.rowPtr = _view(csr.rowPtr, csr.M + 1, np.uint32).copy()
+        self.cols = _view(csr.cols, csr.nnz, np.uint32).copy()
+        self.vals = _view(csr.vals, csr.nnz, np.float32).copy()
+        lib.cute_csr_release(C.byref(csr))
+        self._raw.rowPtr, self._raw.cols, self._raw.vals = _ptr(self.rowPtr, u32p), _ptr(self.cols, u32p), _ptr(self.vals, f32p)
+        self._publish()
+        return self
 
     def as_dict(self):
         return dict(M=self.M, K=self.K, numRowPanels=self.numRowPanels, numBlocks=self.numBlocks,

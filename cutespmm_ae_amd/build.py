@@ -19,7 +19,7 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
           "-pthread"]
 
-LIB_SOURCES = ["host_format.cpp", "host_formats2.cpp", "host_quad.cpp", "gen.cpp", "device.hip"]
+LIB_SOURCES = ["host_format.cpp", "host_formats2.cpp", "host_quad.cpp", "host_cache.cpp", "gen.cpp", "device.hip"]
 
 
 def _run(cmd):

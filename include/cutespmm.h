@@ -97,6 +97,17 @@ int cute_hrpb_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32
 void cute_hrpb_host_release(cute_hrpb_host *h);
 
 /* ------------------------------------------------------------------------------------
+ * host: binary cache of a preprocessed matrix (CSR + canonical HRPB).  No counterpart in the
+ * reference, which rebuilds the format on every run (run.cu:17-20).  Versioned, checksummed;
+ * cute_hrpb_load returns CUTE_ERR_FORMAT for anything that is not a complete file written by
+ * cute_hrpb_save of the same version.  On success `csr` owns the CSR arrays (release with
+ * cute_csr_release) and `h` borrows them and owns the four format arrays (release with
+ * cute_hrpb_host_release, before the CSR).
+ * ---------------------------------------------------------------------------------- */
+int cute_hrpb_save(const cute_hrpb_host *h, const char *path);
+int cute_hrpb_load(const char *path, cute_csr *csr, cute_hrpb_host *h);
+
+/* ------------------------------------------------------------------------------------
  * host: canonical HRPB <-> MFMA-tiled device layout (no reference counterpart for the
  * layout itself; it re-tiles what kernel.cu:16-29 decodes per lane).  Per block one
  * 128-byte header line:

@@ -69,6 +69,29 @@ public:
         : cols(cols_), rowPtr(rowPtr_), vals(vals_), M(M_), K(K_), numRowPanels(M_ / CUTE_TM)
     {
         cute::check(cute_hrpb_build(M, K, rowPtr, cols, vals, &host_), "HRPB");
+        publish(upload);
+    }
+    // Reads what save() wrote (no counterpart in the reference, which rebuilds the format on every
+    // run): the object then owns its CSR arrays as well.
+    explicit HRPB(const char *cache_file, bool upload = true)
+    {
+        cute::check(cute_hrpb_load(cache_file, &owned_csr_, &host_), "HRPB cache file");
+        cols = owned_csr_.cols; rowPtr = owned_csr_.rowPtr; vals = owned_csr_.vals;
+        M = host_.M; K = host_.K; numRowPanels = host_.numRowPanels;
+        publish(upload);
+    }
+    void save(const char *cache_file) const { cute::check(cute_hrpb_save(&host_, cache_file), "HRPB save"); }
+    void freeDevice() { cute_hrpb_dev_free(device); device = nullptr; }   // data.cu:336-339
+    const cute_hrpb_host &host() const { return host_; }
+    ~HRPB() { freeDevice(); cute_hrpb_host_release(&host_); cute_csr_release(&owned_csr_); }
+    HRPB(const HRPB &) = delete;
+    HRPB &operator=(const HRPB &) = delete;
+
+private:
+    cute_hrpb_host host_{};
+    cute_csr owned_csr_{};
+    void publish(bool upload)
+    {
         blocksData = host_.blocksData;
         dataStructSize = host_.numWords;
         num_bricks = host_.numBricks;
@@ -79,17 +102,9 @@ public:
         block_density = num_bricks ? float(numNNZ) / (64.0f * float(num_bricks)) : 0.0f;
         if (upload) {
             int rc = cute_hrpb_upload(&host_, &device);
-            if (rc != CUTE_OK) { cute_hrpb_host_release(&host_); throw cute::Error(rc, "HRPB upload"); }
+            if (rc != CUTE_OK) { cute_hrpb_host_release(&host_); cute_csr_release(&owned_csr_); throw cute::Error(rc, "HRPB upload"); }
         }
     }
-    void freeDevice() { cute_hrpb_dev_free(device); device = nullptr; }   // data.cu:336-339
-    const cute_hrpb_host &host() const { return host_; }
-    ~HRPB() { freeDevice(); cute_hrpb_host_release(&host_); }
-    HRPB(const HRPB &) = delete;
-    HRPB &operator=(const HRPB &) = delete;
-
-private:
-    cute_hrpb_host host_{};
 };
 
 // spmm.cu:258-840

@@ -31,6 +31,14 @@ int main(int argc, char **argv)
                     hrpb.num_bricks, csr.BCSR_nblks, ell.get_ellColIdx_height(), ell.get_ellColIdx_width(), ell.get_num_blocks(),
                     split.get_total_tiles(), split.get_num_heavy_tiles(), split.get_num_heavy_elems(), split.get_num_light_tiles(),
                     split.get_num_light_elems(), diff, small.nnz, small.cols[0]);
+        if (argc > 2) {      // cache file: write, read back, compare every word
+            hrpb.save(argv[2]);
+            HRPB back(argv[2], /*upload=*/false);
+            size_t bad = back.M != hrpb.M || back.K != hrpb.K || back.numNNZ != hrpb.numNNZ || back.dataStructSize != hrpb.dataStructSize;
+            for (unsigned long long i = 0; i < hrpb.dataStructSize && !bad; ++i) bad += back.blocksData[i] != hrpb.blocksData[i];
+            for (unsigned int i = 0; i < hrpb.numNNZ && !bad; ++i) bad += back.cols[i] != hrpb.cols[i] || back.vals[i] != hrpb.vals[i];
+            std::printf("cache=%zu\n", bad);
+        }
         try {
             MTX_READER missing("/nonexistent/file.mtx");
             return 3;

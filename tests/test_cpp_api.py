@@ -17,11 +17,11 @@ def test_reference_style_host_program(cs, orc, tmp_path):
                            "-I", os.path.join(ROOT, "include"), "-L", libdir, "-lcutespmm",
                            "-Wl,-rpath," + libdir, "-o", exe])
     mtx = os.path.join(ROOT, "tests", "golden", "G67.mtx")
-    out = subprocess.run([exe, mtx], check=True, capture_output=True, text=True).stdout.split()
+    out = subprocess.run([exe, mtx, str(tmp_path / "g67.hrpb")], check=True, capture_output=True, text=True).stdout.split()
     got = dict(kv.split("=") for kv in out)
     M, K, nnz, rp, cl, vl = orc.mtx_read(mtx)
     h = orc.hrpb_build(M, K, rp, cl, vl)
     assert (int(got["M"]), int(got["K"]), int(got["nnz"])) == (M, K, nnz)
     assert (int(got["panels"]), int(got["blocks"]), int(got["words"])) == (h["numRowPanels"], h["numBlocks"], h["numWords"])
     assert got["bcsr"] == "8750" and got["tiles"] == "4325" and got["heavy"] == "1875/33800" and got["light"] == "2450/6200"
-    assert got["densediff"] == "0" and got["grown"] == "2,1"
+    assert got["densediff"] == "0" and got["grown"] == "2,1" and got["cache"] == "0"

@@ -234,3 +234,25 @@ def test_plan_rejects_bad_arguments(cs, torch_cuda):
     plan = cs.SPMM_TC(h, 32)
     with pytest.raises(ValueError):
         plan.run(torch.zeros((32, 16), device="cuda"), torch.zeros((32, 32), device="cuda"))
+
+
+def test_driver_and_sweep_tool(cs, torch_cuda, tmp_path):
+    """The C++ driver (counterpart of run.cu's main) on the golden matrix, through the sweep tool:
+    three widths, results checked by the driver itself against the plain CSR kernel, and a second
+    pass that reads the converted matrix from the cache file."""
+    import os
+    from cutespmm_ae_amd import sweep
+    from test_oracle_pins import GOLD
+    mtx = os.path.join(GOLD, "G67.mtx")
+    cache = str(tmp_path / "g67.hrpb")
+    first = sweep.run_one(mtx, [32, 128, 512], 5, cache)
+    again = sweep.run_one(mtx, [32, 128, 512], 5, cache)
+    assert [r["N"] for r in first] == [32, 128, 512] and os.path.getsize(cache) > 0
+    for a, b in zip(first, again):
+        assert not a["from_cache"] and b["from_cache"]
+        assert (a["M"], a["K"], a["nnz"], a["blocks"], a["bricks"]) == (10000, 10000, 40000, 2500, b["bricks"])
+        assert (b["M"], b["nnz"], b["blocks"]) == (10000, 40000, 2500)
+        for r in (a, b):
+            assert r["gflops"] > 0 and r["max_rel_err"] <= 1e-5 and r["backward_err"] <= BERR
+    text = sweep.table([("G67", r) for r in first])
+    assert text.splitlines()[0] == "matrix, N(feature size), cuTeSpMM GFLOPS, CSR GFLOPS" and len(text.splitlines()) == 4
