@@ -31,6 +31,7 @@ ABI_SYMBOLS = [
     "cute_coo_read", "cute_coo_save_mtx", "cute_coo_release", "cute_coo_to_csr", "cute_csr_i32_release",
     "cute_csr_to_dense", "cute_csr_count_blocks", "cute_csr_to_bcsr", "cute_bcsr_release",
     "cute_blocked_ell_build", "cute_blocked_ell_to_dense", "cute_blocked_ell_release",
+    "cute_blocked_ell_upload", "cute_blocked_ell_dev_free", "cute_blocked_ell_spmm",
     "cute_splitter_split", "cute_split_release", "cute_classify_blocks", "cute_sequential_spmm",
 ]
 
@@ -153,6 +154,10 @@ def load_library():
     lib.cute_quad_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.argtypes = [C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.restype = None
+    lib.cute_blocked_ell_upload.argtypes = [C.POINTER(cute_blocked_ell), C.POINTER(C.c_void_p)]
+    lib.cute_blocked_ell_dev_free.argtypes = [C.c_void_p]
+    lib.cute_blocked_ell_dev_free.restype = None
+    lib.cute_blocked_ell_spmm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int, C.c_void_p]
     lib.cute_hrpb_save.argtypes = [C.POINTER(cute_hrpb_host), C.c_char_p]
     lib.cute_hrpb_load.argtypes = [C.c_char_p, C.POINTER(cute_csr), C.POINTER(cute_hrpb_host)]
     lib.cute_partition.restype = C.c_int64
@@ -563,6 +568,19 @@ def csr_spmm_dev(alg, hrpb, MatB, MatC, stream=None):
     return MatC
 
 
+def csr_spmm_tensors(alg, rowPtr, cols, vals, MatB, MatC, stream=None):
+    """The plain CSR kernels on caller-owned GPU tensors: rowPtr/cols int32 (or uint32 bits), vals float32."""
+    import torch
+    for t in (rowPtr, cols):
+        if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
+            raise TypeError("rowPtr and cols must be contiguous int32 tensors on the GPU")
+    M = int(rowPtr.numel()) - 1
+    _check(load_library().cute_csr_spmm_dev(int(alg), C.c_void_p(rowPtr.data_ptr()), C.c_void_p(cols.data_ptr()),
+                                            _dev_ptr(vals), _dev_ptr(MatB), _dev_ptr(MatC), M, int(MatB.shape[1]),
+                                            _stream_ptr(stream)), "cute_csr_spmm_dev")
+    return MatC
+
+
 def GPU_CSR_cuSPARSE_NEW(rowPtr, cols, vals, nnz, hB, hC, m, k, n, iters, alg=2):
     """Host arrays in, host C out, returns ms per launch (signature of spmm.cu:860-861)."""
     rowPtr, cols, vals = _as(rowPtr, np.uint32), _as(cols, np.uint32), _as(vals, np.float32)
@@ -713,13 +731,44 @@ class preprocess:
     def get_num_blocks(self): return self._nb
     def get_num_elems(self): return self._ne
 
+    def _raw(self):
+        return cute_blocked_ell(self.BlockSize, self._h, self._w, self._nb, self._ne, _ptr(self._idx, i32p),
+                                _ptr(self._val, f32p))
+
+    def spmm(self, MatB, MatC, accumulate=False, stream=None):
+        """MatC[height*BlockSize, N] (+)= ELL . MatB[ncols, N] on the GPU (float32 tensors); the device
+        copy of the format is made on first use."""
+        if getattr(self, "_dev", None) is None:
+            dev, raw = C.c_void_p(), self._raw()
+            _check(load_library().cute_blocked_ell_upload(C.byref(raw), C.byref(dev)), "cute_blocked_ell_upload")
+            self._dev = _DevGuard(dev, "cute_blocked_ell_dev_free")
+        N = int(MatB.shape[1])
+        if tuple(MatB.shape) != (self._ncols, N) or tuple(MatC.shape) != (self._h * self.BlockSize, N):
+            raise ValueError("MatB must be [%d,N] and MatC [%d,N]" % (self._ncols, self._h * self.BlockSize))
+        _check(load_library().cute_blocked_ell_spmm(self._dev.handle, _dev_ptr(MatB), _dev_ptr(MatC), N,
+                                                    int(bool(accumulate)), _stream_ptr(stream)), "cute_blocked_ell_spmm")
+        return MatC
+
     def blockedELLToDense(self):
         dense = np.zeros((self._h * self.BlockSize, self._ncols), np.float32)
-        raw = cute_blocked_ell(self.BlockSize, self._h, self._w, self._nb, self._ne, _ptr(self._idx, i32p),
-                               _ptr(self._val, f32p))
+        raw = self._raw()
         _check(load_library().cute_blocked_ell_to_dense(C.byref(raw), self._ncols, _ptr(dense, f32p)),
                "cute_blocked_ell_to_dense")
         return dense
+
+
+class _DevGuard:
+    """Frees a device handle of the library when the last owner goes."""
+
+    def __init__(self, handle, free_name):
+        self.handle, self._free = handle, free_name
+
+    def __del__(self):
+        try:
+            if self.handle:
+                getattr(load_library(), self._free)(self.handle)
+        except Exception:
+            pass
 
 
 class Splitter:

@@ -500,6 +500,27 @@ int time_launches(hipStream_t s, int warmup, int iters, float *ms_out, Launch la
 }
 }  // namespace
 
+struct cute_blocked_ell_dev {
+    int32_t blockSize = 0, height = 0, width = 0;
+    int32_t *dColIdx = nullptr;
+    float *dValues = nullptr;
+};
+
+namespace {
+template <int VEC, bool ACC>
+void launch_blocked_ell(const cute_blocked_ell_dev *d, const float *dB, float *dC, uint32_t N, hipStream_t s)
+{
+    const uint32_t rows = uint32_t(d->height) * uint32_t(d->blockSize), strips = rows / 16u;
+    const dim3 grid((strips + 3u) / 4u, (N + 16u * VEC - 1u) / (16u * VEC)), block(256);
+    if (N % (16u * VEC) == 0)
+        hipLaunchKernelGGL((cute_dev::blocked_ell_f32<VEC, true, ACC>), grid, block, 0, s, d->dColIdx, d->dValues,
+                           uint32_t(d->blockSize), uint32_t(d->width), strips, rows, dB, dC, N);
+    else
+        hipLaunchKernelGGL((cute_dev::blocked_ell_f32<VEC, false, ACC>), grid, block, 0, s, d->dColIdx, d->dValues,
+                           uint32_t(d->blockSize), uint32_t(d->width), strips, rows, dB, dC, N);
+}
+}  // namespace
+
 extern "C" {
 
 // Replaces SPMM_TC::run (spmm.cu:823-839): picks the kernel instantiation from N and
@@ -544,6 +565,55 @@ int cute_csr_spmm_dev(int alg, const uint32_t *dRowPtr, const uint32_t *dCols, c
     const DeviceContext &c = context();
     if (c.status != CUTE_OK) return c.status;
     return csr_launch(alg, dRowPtr, dCols, dVals, dB, dC, M, N, static_cast<hipStream_t>(stream));
+}
+
+
+void cute_blocked_ell_dev_free(cute_blocked_ell_dev *d)
+{
+    if (!d) return;
+    (void)hipFree(d->dColIdx);
+    (void)hipFree(d->dValues);
+    delete d;
+}
+
+int cute_blocked_ell_upload(const cute_blocked_ell *e, cute_blocked_ell_dev **out)
+{
+    if (!e || !out || e->blockSize <= 0 || e->height < 0 || e->width < 0) return CUTE_ERR_ARG;
+    *out = nullptr;
+    if (e->blockSize % 16) return CUTE_ERR_SHAPE;        // the kernel walks 16 x 16 tiles
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    cute_blocked_ell_dev *d = new cute_blocked_ell_dev;
+    d->blockSize = e->blockSize; d->height = e->height; d->width = e->width;
+    const uint64_t cells = uint64_t(e->height) * uint64_t(e->width);
+    int rc = upload(&d->dColIdx, e->ellColIdx, cells);
+    if (rc == CUTE_OK) rc = upload(&d->dValues, e->ellValues, cells * uint64_t(e->blockSize) * uint64_t(e->blockSize));
+    if (rc != CUTE_OK) { cute_blocked_ell_dev_free(d); return rc; }
+    *out = d;
+    return CUTE_OK;
+}
+
+
+// C[height*blockSize x N] (+)= ELL . B[ncols x N], device pointers, asynchronous on `stream`.
+int cute_blocked_ell_spmm(const cute_blocked_ell_dev *d, const float *dB, float *dC, uint32_t N, int accumulate, void *stream)
+{
+    if (!d || !dB || !dC) return CUTE_ERR_ARG;
+    if (N == 0) return CUTE_ERR_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC)) & 15u) return CUTE_ERR_ARG;
+    if (d->height == 0) return CUTE_OK;
+    if ((N + 15u) / 16u > 65535u) return CUTE_ERR_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    if (accumulate) {
+        if (vec == 4) launch_blocked_ell<4, true>(d, dB, dC, N, s);
+        else if (vec == 2) launch_blocked_ell<2, true>(d, dB, dC, N, s);
+        else launch_blocked_ell<1, true>(d, dB, dC, N, s);
+    } else {
+        if (vec == 4) launch_blocked_ell<4, false>(d, dB, dC, N, s);
+        else if (vec == 2) launch_blocked_ell<2, false>(d, dB, dC, N, s);
+        else launch_blocked_ell<1, false>(d, dB, dC, N, s);
+    }
+    return check_launch("blocked-ELL launch");
 }
 
 // Shape of GPU_CSR_cuSPARSE_NEW (spmm.cu:860-960): host arrays in, host C out, one warm-up

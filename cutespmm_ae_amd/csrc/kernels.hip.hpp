@@ -526,6 +526,69 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Blocked-ELL SpMM (the format of inc/prepareBlkEll.hpp): dense blockSize x blockSize blocks,
+// ellColIdx[height x width] block-column ids (ascending, -1 padded), ellValues row-major
+// [height*blockSize x width*blockSize].  One wavefront per (16-row strip, slab of 16*VEC columns).
+// A 16x16 tile of A is one 16-byte load per lane: lane (row = L%16, q = L/16) holds
+// A[row][4q..4q+3].  MFMA number e of the tile takes element e of that vector, i.e. k index
+// 4q+e from lane group q -- so lane group q fetches B rows 4q+e, e = 0..3, itself, and no
+// cross-lane move is needed.  Accumulator layout and the column interleave that gives every
+// lane VEC consecutive C columns are those of the brick kernel.
+// ACCUMULATE: C += A.B (for the heavy part of a split matrix), else C = A.B.
+// ---------------------------------------------------------------------------------------
+template <int VEC, bool FULL, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict__ ell_col, const float *__restrict__ ell_val,
+                                                       uint32_t block_size, uint32_t width, uint32_t num_strips,
+                                                       uint32_t num_rows, const float *__restrict__ B, float *__restrict__ C,
+                                                       uint32_t N)
+{
+    typedef typename Vec<VEC>::type V;
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t strip = blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+    if (strip >= num_strips) return;
+    const uint32_t row16 = lane & 15u, q = lane >> 4;
+    const uint32_t c0 = blockIdx.y * (16u * VEC) + row16 * VEC;       // this lane's VEC columns of the slab
+    const bool col_live = FULL || c0 < N;
+    const uint32_t block_row = (strip * 16u) / block_size;
+    const size_t pitch = size_t(width) * block_size;
+    const float *a_row = ell_val + size_t(strip * 16u + row16) * pitch + q * 4u;
+    const int32_t *cols = ell_col + size_t(block_row) * width;
+
+    f32x4 acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = f32x4(0.0f);
+
+    for (uint32_t w = 0; w < width; ++w) {
+        const int32_t bc = cols[w];
+        if (bc < 0) break;                                            // padding follows the last block
+        for (uint32_t kt = 0; kt < block_size; kt += 16u) {           // 16-wide k tiles of the block
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(a_row + size_t(w) * block_size + kt);
+            const float *b_row = B + size_t(uint32_t(bc) * block_size + kt + q * 4u) * N + c0;
+            V b[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[e] = col_live ? *reinterpret_cast<const V *>(b_row + size_t(e) * N) : V(0.0f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v)
+                    acc[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], vec_get<VEC>(b[e], v), acc[v], 0, 0, 0);
+        }
+    }
+    if (!col_live) return;
+    const uint32_t r0 = strip * 16u + q * 4u;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (r0 + r >= num_rows) break;
+        V *dst = reinterpret_cast<V *>(C + size_t(r0 + r) * N + c0);
+        V out;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[v][r]);
+        if (ACCUMULATE) out += *dst;
+        *dst = out;
+    }
+}
+
 // Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).
 __global__ void zero_panels(const uint32_t *__restrict__ panels, uint32_t count, float *__restrict__ C, uint32_t N)
 {

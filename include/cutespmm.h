@@ -238,6 +238,16 @@ int cute_blocked_ell_build(const cute_csr_i32 *csr, int32_t blockSize, cute_bloc
 int cute_blocked_ell_to_dense(const cute_blocked_ell *e, int32_t ncols, float *dense);
 void cute_blocked_ell_release(cute_blocked_ell *e);
 
+/* Device twin and SpMM of a Blocked-ELL matrix: C[height*blockSize x N] = ELL . B[ncols x N]
+ * (accumulate != 0: C += ...), fp32 MFMA on the dense blocks.  Stands where the reference's harness
+ * calls cusparseSpMM on a CUSPARSE_FORMAT_BLOCKED_ELL descriptor (gpu_kernels.cu:166-223).
+ * blockSize must be a multiple of 16; B and C are device pointers, 16-byte aligned. */
+typedef struct cute_blocked_ell_dev cute_blocked_ell_dev;
+int cute_blocked_ell_upload(const cute_blocked_ell *e, cute_blocked_ell_dev **out);
+void cute_blocked_ell_dev_free(cute_blocked_ell_dev *d);
+int cute_blocked_ell_spmm(const cute_blocked_ell_dev *d, const float *dB, float *dC, uint32_t N, int accumulate,
+                          void *stream);
+
 typedef struct cute_split {        /* Splitter, inc/splitter.hpp:14-187                                  */
     int32_t totalTiles, numHeavyTiles, numHeavyElems, numLightTiles, numLightElems;
     cute_coo heavy, light;                  /* tile nnz >= threshold / < threshold; CSR order kept     */

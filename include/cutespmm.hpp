@@ -258,8 +258,15 @@ public:
     {
         cute::check(cute_blocked_ell_build(&A_CSR->raw(), BlockSize, &e_), "preprocess");
     }
-    ~preprocess() { cute_blocked_ell_release(&e_); }
+    ~preprocess() { cute_blocked_ell_dev_free(dev_); cute_blocked_ell_release(&e_); }
     void blockedELLToDense(DType *dense) { cute::check(cute_blocked_ell_to_dense(&e_, ncols_, dense), "blockedELLToDense"); }
+    // C[height*BlockSize x N] (+)= ELL . B[ncols x N] on the GPU, device pointers; the place of the
+    // cusparseSpMM call on a Blocked-ELL descriptor in the reference's harness (gpu_kernels.cu:166-223).
+    void spmm(const DType *dB, DType *dC, unsigned int N, bool accumulate = false, void *stream = nullptr)
+    {
+        if (!dev_) cute::check(cute_blocked_ell_upload(&e_, &dev_), "Blocked-ELL upload");
+        cute::check(cute_blocked_ell_spmm(dev_, dB, dC, N, accumulate ? 1 : 0, stream), "Blocked-ELL SpMM");
+    }
     int *get_ellColIdx() { return e_.ellColIdx; }
     int get_ellColIdx_height() { return e_.height; }
     int get_ellColIdx_width() { return e_.width; }
@@ -271,6 +278,7 @@ public:
 
 private:
     cute_blocked_ell e_{};
+    cute_blocked_ell_dev *dev_ = nullptr;
     int ncols_;
 };
 

@@ -256,3 +256,64 @@ def test_driver_and_sweep_tool(cs, torch_cuda, tmp_path):
             assert r["gflops"] > 0 and r["max_rel_err"] <= 1e-5 and r["backward_err"] <= BERR
     text = sweep.table([("G67", r) for r in first])
     assert text.splitlines()[0] == "matrix, N(feature size), cuTeSpMM GFLOPS, CSR GFLOPS" and len(text.splitlines()) == 4
+
+
+@pytest.mark.parametrize("block_size", [16, 32])
+def test_blocked_ell_spmm(cs, orc, torch_cuda, block_size):
+    """Blocked-ELL device SpMM against the CSR oracle: random values (tolerance), integer values
+    (bit for bit), every vector width of N, and C += on top of a previous result."""
+    torch = torch_cuda
+    rng = np.random.default_rng(40 + block_size)
+    M, K = 192, 256
+    for values, Ns in (("normal", (1, 6, 64, 100, 128)), ("ints", (32,))):
+        rp, cl, vl = random_csr(rng, M, K, density=0.06, empty_rows=set(range(64, 96)), values=values)
+        csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp.astype(np.int32), cols=cl.astype(np.int32), values=vl)
+        ell = cs.preprocess(csr, block_size)
+        assert ell.get_ellColIdx_height() * block_size == M
+        for N in Ns:
+            B = (rng.integers(-4, 5, (K, N)) if values == "ints" else rng.standard_normal((K, N))).astype(np.float32)
+            ref = orc.spmm_csr(rp, cl, vl, B)
+            dB = torch.from_numpy(B).cuda()
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            ell.spmm(dB, dC)
+            torch.cuda.synchronize()
+            out = dC.cpu().numpy()
+            if values == "ints":
+                assert (out == ref).all()
+            else:
+                assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (block_size, N)
+            ell.spmm(dB, dC, accumulate=True)
+            torch.cuda.synchronize()
+            twice = dC.cpu().numpy()
+            assert np.allclose(twice, 2 * out, rtol=1e-6, atol=0) if values != "ints" else (twice == 2 * ref).all()
+
+
+def test_split_matrix_spmm(cs, orc, torch_cuda):
+    """Splitter: heavy tiles through the Blocked-ELL kernel, light tiles through the CSR kernel,
+    added into one C -- equal to the product with the unsplit matrix."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    M = K = 256
+    N = 64
+    D = np.zeros((M, K), np.float32)
+    D[rng.random((M, K)) < 0.01] = 1.0                      # light background
+    for t in rng.choice(256, 40, replace=False):            # some dense 16x16 tiles
+        r, c = (t // 16) * 16, (t % 16) * 16
+        D[r:r + 16, c:c + 16] = (rng.random((16, 16)) < 0.7)
+    D *= rng.integers(1, 4, D.shape)
+    rp, cl, vl = csr_from_dense(D)
+    csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp.astype(np.int32), cols=cl.astype(np.int32), values=vl)
+    sp = cs.Splitter(csr, 16, 64)
+    assert sp.get_num_heavy_tiles() > 0 and sp.get_num_light_tiles() > 0
+    heavy, light = cs.CSR_Matrix(sp.get_heavyMatrix()), cs.CSR_Matrix(sp.get_lightMatrix())
+    assert heavy.nnz + light.nnz == len(vl)
+    B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    dB = torch.from_numpy(B).cuda()
+    dC = torch.full((M, N), float("nan"), device="cuda")
+    lp = torch.from_numpy(light.rowPtr.astype(np.int32)).cuda()
+    lc = torch.from_numpy(light.cols.astype(np.int32)).cuda()
+    lv = torch.from_numpy(light.values).cuda()
+    cs.csr_spmm_tensors(2, lp, lc, lv, dB, dC)               # C = light . B
+    cs.preprocess(heavy, 16).spmm(dB, dC, accumulate=True)   # C += heavy . B
+    torch.cuda.synchronize()
+    assert (dC.cpu().numpy() == orc.spmm_csr(rp, cl, vl, B)).all()
