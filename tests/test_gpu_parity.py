@@ -317,3 +317,26 @@ def test_split_matrix_spmm(cs, orc, torch_cuda):
     cs.preprocess(heavy, 16).spmm(dB, dC, accumulate=True)   # C += heavy . B
     torch.cuda.synchronize()
     assert (dC.cpu().numpy() == orc.spmm_csr(rp, cl, vl, B)).all()
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("cfg", [3, 4, 5])
+def test_full_size_other_configs(cs, orc, torch_cuda, cfg):
+    """The other benchmark workloads at full size through the planner's own choice: comparison with
+    the oracle, and the column-sum identity 1^T C = (1^T A) B, which does not depend on the oracle."""
+    torch = torch_cuda
+    A = cs.gen_config(cfg)
+    N = cs.CONFIGS[cfg]["N"]
+    B = cs.gen_dense(cs.SEED_BASE + 100 + cfg, A.K, N, 2)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    out, plan = _run(cs, torch, h, B)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+    assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, out) <= BERR, plan.info
+    colsum = np.zeros(A.K, np.float64)
+    np.add.at(colsum, A.cols.astype(np.int64), A.vals.astype(np.float64))
+    scale = np.zeros(A.K, np.float64)
+    np.add.at(scale, A.cols.astype(np.int64), np.abs(A.vals.astype(np.float64)))
+    expect = colsum @ B.astype(np.float64)
+    bound = scale @ np.abs(B.astype(np.float64))
+    got = out.sum(0, dtype=np.float64)
+    assert (np.abs(got - expect) <= 1e-5 * bound).all()
