@@ -21,10 +21,10 @@ ABI_SYMBOLS = [
     "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
-    "cute_quad_build", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
+    "cute_quad_build", "cute_quad_build_strips", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
-    "cute_hrpb_upload", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
+    "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
     "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run",
     "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
     "cute_device_info",
@@ -68,7 +68,8 @@ class cute_hrpb_tiled(C.Structure):
 
 class cute_quad_lists(C.Structure):
     _fields_ = [("M", C.c_uint32), ("K", C.c_uint32), ("numRowPanels", C.c_uint32), ("numGroups", C.c_uint64),
-                ("groupPtr", u32p), ("cols", u32p), ("vals", f32p)]
+                ("groupPtr", u32p), ("cols", u32p), ("vals", f32p), ("tail", u32p), ("numPairs", C.c_uint64),
+                ("rowsPerList", C.c_uint32)]
 
 
 class cute_tunables(C.Structure):
@@ -152,6 +153,8 @@ def load_library():
     lib.cute_hrpb_untile.argtypes = [C.POINTER(cute_hrpb_tiled), C.POINTER(cute_hrpb_host)]
     lib.cute_hrpb_tiled_release.argtypes = [C.POINTER(cute_hrpb_tiled)]
     lib.cute_quad_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_quad_lists)]
+    lib.cute_quad_build_strips.argtypes = lib.cute_quad_build.argtypes
+    lib.cute_hrpb_upload_layout.argtypes = [C.POINTER(cute_hrpb_host), C.c_int, C.POINTER(C.c_void_p)]
     lib.cute_quad_release.argtypes = [C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.restype = None
     lib.cute_blocked_ell_upload.argtypes = [C.POINTER(cute_blocked_ell), C.POINTER(C.c_void_p)]
@@ -427,9 +430,12 @@ class HRPB:
         lib.cute_hrpb_host_release(C.byref(back))
         return out
 
-    def upload(self):
+    def upload(self, quad_layout=0):
+        """Device twin (made once).  quad_layout: 0 library's choice, 1 lockstep lists per panel,
+        2 one list per 4-row strip; only the first call's choice counts."""
         if not self._dev:
-            _check(load_library().cute_hrpb_upload(C.byref(self._raw), C.byref(self._dev)), "cute_hrpb_upload")
+            _check(load_library().cute_hrpb_upload_layout(C.byref(self._raw), int(quad_layout), C.byref(self._dev)),
+                   "cute_hrpb_upload_layout")
         return self._dev
 
     def device_bytes(self):
@@ -481,16 +487,18 @@ def _dev_ptr(t):
     return C.c_void_p(t.data_ptr())
 
 
-def quad_lists(M, K, rowPtr, cols, vals):
+def quad_lists(M, K, rowPtr, cols, vals, strips=False):
     """Host copy of the 4x4x1 MFMA kernel's layout built from a CSR matrix:
-    dict(groupPtr[P+1], cols[G,16], vals[G,64])."""
+    dict(groupPtr[U+1], cols[G,16], vals[G,64], tail[U], numPairs, rowsPerList); U = 16-row panels,
+    or 4-row strips with ``strips=True``."""
     rowPtr = np.ascontiguousarray(rowPtr, np.uint32)
     cols = np.ascontiguousarray(cols, np.uint32)
     vals = np.ascontiguousarray(vals, np.float32)
     q = cute_quad_lists()
-    _check(load_library().cute_quad_build(int(M), int(K), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p),
-                                          C.byref(q)), "cute_quad_build")
-    out = dict(numGroups=int(q.numGroups),
+    build = load_library().cute_quad_build_strips if strips else load_library().cute_quad_build
+    _check(build(int(M), int(K), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p), C.byref(q)), "cute_quad_build")
+    out = dict(numGroups=int(q.numGroups), numPairs=int(q.numPairs), rowsPerList=int(q.rowsPerList),
+               tail=_view(q.tail, q.numRowPanels, np.uint32).copy(),
                groupPtr=_view(q.groupPtr, q.numRowPanels + 1, np.uint32).copy(),
                cols=_view(q.cols, q.numGroups * 16, np.uint32).reshape(-1, 16).copy(),
                vals=_view(q.vals, q.numGroups * 64, np.float32).reshape(-1, 64).copy())

@@ -83,6 +83,8 @@ struct cute_hrpb_dev {
     uint64_t numGroups = 0;
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
     std::vector<uint32_t> qgp;          // host copy of the quad lists' groupPtr
+    uint32_t quadRows = CUTE_TM;        // rows per list unit: 16 (lockstep lists per panel) or 4 (strips)
+    uint64_t quadPairs = 0;             // occupied (row group, column) pairs
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
     std::vector<uint32_t> panelCols;    // active columns per row panel
     std::vector<uint32_t> panelMaxRow;  // longest row of each panel
@@ -99,6 +101,7 @@ struct cute_spmm_plan {
     uint4 *dChunks = nullptr;
     uint32_t *dAtomicPanels = nullptr;
     uint32_t numAtomicPanels = 0;
+    uint32_t atomicPanelRows = CUTE_TM; // rows of one entry of dAtomicPanels
     uint32_t *dRowList = nullptr;
     uint32_t numRows = 0;
 };
@@ -132,9 +135,11 @@ void cute_hrpb_dev_free(cute_hrpb_dev *d)
 
 uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d) { return d ? d->bytes : 0; }
 
-int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
+int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out) { return cute_hrpb_upload_layout(h, 0, out); }
+
+int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_dev **out)
 {
-    if (!h || !out || !h->rowPtr) return CUTE_ERR_ARG;
+    if (!h || !out || !h->rowPtr || quad_layout < 0 || quad_layout > 2) return CUTE_ERR_ARG;
     *out = nullptr;
     const DeviceContext &c = context();
     if (c.status != CUTE_OK) return c.status;
@@ -185,10 +190,19 @@ int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out)
                uint64_t(h->nnz) * 8;
     cute_hrpb_tiled_release(&t);
     if (rc == CUTE_OK) {
+        // Lockstep lists unless they would be mostly padding (a few very long rows stretch the
+        // lists of their neighbours): then one list per 4-row strip.
         cute_quad_lists ql;
-        rc = cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
+        rc = quad_layout == 2 ? cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql)
+                              : cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
+        if (rc == CUTE_OK && quad_layout == 0 && ql.numGroups && double(ql.numPairs) < 0.6 * 16.0 * double(ql.numGroups)) {
+            cute_quad_release(&ql);
+            rc = cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
+        }
         if (rc == CUTE_OK) {
             d->numGroups = ql.numGroups;
+            d->quadRows = ql.rowsPerList;
+            d->quadPairs = ql.numPairs;
             d->qgp.assign(ql.groupPtr, ql.groupPtr + ql.numRowPanels + 1);
             rc = upload(&d->dQCols, ql.cols, ql.numGroups * 16);
             if (rc == CUTE_OK) rc = upload(&d->dQVals, ql.vals, ql.numGroups * 64);
@@ -312,24 +326,28 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // of the whole job (and at least 8 blocks), into pieces of about that share.
     // work units along a panel: 16-column blocks for the brick kernel, groups for the quad kernel
     const std::vector<uint32_t> &unit = p->shape == 2 ? d->qgp : d->brp;
+    // units per panel: 4 when the quad lists are kept per 4-row strip
+    const uint32_t upp = (p->shape == 2 && d->quadRows == 4) ? 4u : 1u;
+    const uint32_t num_units = d->P * upp;
     const uint32_t resident = uint32_t(c.num_cus) * 4u * 8u;   // 4 SIMDs x 8 wavefronts per CU
     const uint32_t slots = t.slots ? t.slots : resident;
     std::vector<uint32_t> quads;
     if (t.slots) {
-        int64_t n = cute_partition(d->P, unit.data(), num_slabs, slots, nullptr, 0);
+        int64_t n = cute_partition(num_units, unit.data(), num_slabs, slots, nullptr, 0);
         if (n < 0) { delete p; return int(n); }
         quads.resize(uint64_t(n) * 4);
-        cute_partition(d->P, unit.data(), num_slabs, slots, quads.data(), uint64_t(n));
+        cute_partition(num_units, unit.data(), num_slabs, slots, quads.data(), uint64_t(n));
     } else {
         uint64_t work = 0;
-        for (uint32_t q = 0; q < d->P; ++q)
-            if (!to_rows[q]) work += unit[q + 1] - unit[q];
-        const uint64_t mean = n_brick ? (work + n_brick - 1) / n_brick : 1;
+        uint64_t busy = 0;
+        for (uint32_t q = 0; q < num_units; ++q)
+            if (!to_rows[q / upp] && unit[q + 1] != unit[q]) { work += unit[q + 1] - unit[q]; ++busy; }
+        const uint64_t mean = busy ? (work + busy - 1) / busy : 1;
         const uint64_t share = (work * num_slabs + resident - 1) / resident;
         const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, mean), 8));
-        for (uint32_t q = 0; q < d->P; ++q) {
+        for (uint32_t q = 0; q < num_units; ++q) {
             const uint32_t s = unit[q], e = unit[q + 1];
-            if (s == e || to_rows[q]) continue;
+            if (s == e || to_rows[q / upp]) continue;
             const uint32_t nblk = e - s;
             if (nblk <= 2 * target) {
                 quads.insert(quads.end(), {s, e, q, 0u});
@@ -346,7 +364,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     for (size_t i = 0; i + 3 < quads.size(); i += 4) {
         const uint32_t s = quads[i], e = quads[i + 1], pan = quads[i + 2];
         uint32_t atomic = quads[i + 3];
-        if (to_rows[pan]) continue;
+        if (to_rows[pan / upp]) continue;
         const uint32_t len = e - s;
         const uint32_t cap = t.max_chunk_blocks ? t.max_chunk_blocks : len;
         if (len > cap) atomic = 1;                 // cut further than the partition asked for
@@ -357,6 +375,10 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             n_atomic += atomic;
         }
     }
+    // a strip without pairs inside an MFMA-routed panel still has to be written (as zeros): an empty chunk
+    if (upp > 1)
+        for (uint32_t q = 0; q < num_units; ++q)
+            if (unit[q] == unit[q + 1] && !to_rows[q / upp]) chunks.push_back(make_uint4(unit[q], unit[q], q, 0u));
     // panels ascend through the chunk list, so each atomic panel is listed (and zeroed) once
     std::vector<uint32_t> row_list;
     for (uint32_t q = 0; q < d->P; ++q)
@@ -368,6 +390,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
     p->numAtomicPanels = uint32_t(atomic_panels.size());
+    p->atomicPanelRows = CUTE_TM / upp;
     p->numRows = uint32_t(row_list.size());
     p->info.N = N;
     p->info.slabWidth = slab;
@@ -533,18 +556,21 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
     const uint32_t N = p->info.N;
     if (p->numAtomicPanels) {
         hipLaunchKernelGGL(cute_dev::zero_panels, dim3(p->numAtomicPanels), dim3(256), 0, s, p->dAtomicPanels,
-                           p->numAtomicPanels, dC, N);
+                           p->numAtomicPanels, p->atomicPanelRows, dC, N);
     }
     if (p->info.numChunks && p->shape == 2) {
         const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
         const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
-        if (N % 64u == 0)
-            hipLaunchKernelGGL(cute_dev::hrpb_quad_f32<true>, grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,
-                               p->d->dQCols, p->d->dQVals, dB, dC, N);
-        else
-            hipLaunchKernelGGL(cute_dev::hrpb_quad_f32<false>, grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,
-                               p->d->dQCols, p->d->dQVals, dB, dC, N);
+        const bool full = N % 64u == 0, strips = p->d->quadRows == 4;
+#define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
+    hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,        \
+                       p->d->dQCols, p->d->dQVals, dB, dC, N)
+        if (full && strips) CUTE_QUAD_LAUNCH(true, true);
+        else if (full) CUTE_QUAD_LAUNCH(true, false);
+        else if (strips) CUTE_QUAD_LAUNCH(false, true);
+        else CUTE_QUAD_LAUNCH(false, false);
+#undef CUTE_QUAD_LAUNCH
     } else if (p->info.numChunks) {
         if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
         else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);

@@ -58,6 +58,7 @@ void cute_quad_release(cute_quad_lists *q)
     std::free(q->groupPtr);
     std::free(q->cols);
     std::free(q->vals);
+    std::free(q->tail);
     std::memset(q, 0, sizeof(*q));
 }
 
@@ -70,17 +71,24 @@ int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32
     out->M = M;
     out->K = K;
     out->numRowPanels = P;
+    out->rowsPerList = CUTE_TM;
     out->groupPtr = cute::alloc_array<uint32_t>(uint64_t(P) + 1);
-    if (!out->groupPtr) return CUTE_ERR_NOMEM;
+    out->tail = cute::alloc_array<uint32_t>(P);
+    if (!out->groupPtr || !out->tail) { cute_quad_release(out); return CUTE_ERR_NOMEM; }
+    std::vector<uint64_t> pairs_of(P, 0);
 
     // sweep 1: groups per panel = ceil(longest of the four lists / 4)
     cute::parallel_ranges(P, 64, [&](uint64_t b, uint64_t e, unsigned) {
         for (uint64_t q = b; q < e; ++q) {
             uint32_t longest = 0;
-            for (uint32_t rg = 0; rg < 4; ++rg)
-                longest = std::max(longest, merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * CUTE_TM + rg * 4,
-                                                            [](uint32_t, const float *) {}));
+            for (uint32_t rg = 0; rg < 4; ++rg) {
+                const uint32_t len = merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * CUTE_TM + rg * 4,
+                                                     [](uint32_t, const float *) {});
+                longest = std::max(longest, len);
+                pairs_of[q] += len;
+            }
             out->groupPtr[q + 1] = (longest + 3) / 4;
+            out->tail[q] = longest ? 4u * (longest - 4u * ((longest + 3) / 4 - 1)) : 0u;   // pair slots in use in the last group
         }
     });
     uint64_t total = 0;
@@ -90,6 +98,7 @@ int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32
         out->groupPtr[q + 1] = uint32_t(total);
     }
     out->numGroups = total;
+    for (uint32_t q = 0; q < P; ++q) out->numPairs += pairs_of[q];
     out->cols = cute::alloc_array<uint32_t>(total * 16);
     out->vals = cute::alloc_array<float>(total * 64);     // calloc: absent entries are +0.0f
     if (!out->cols || !out->vals) { cute_quad_release(out); return CUTE_ERR_NOMEM; }
@@ -112,6 +121,60 @@ int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32
                 });
                 for (; s < steps; ++s) out->cols[(g0 + s / 4) * 16 + 4 * (s % 4) + rg] = last;
             }
+        }
+    });
+    return CUTE_OK;
+}
+
+// The same pairs with one list per 4-row strip instead of four lockstep lists per panel: nothing
+// is padded to a longer neighbour, which is what a matrix with a few very long rows needs (the
+// strip holding such a row would otherwise stretch the other three of its panel).  A group is 16
+// consecutive pairs of one strip: cols[g*16 + p], vals[g*64 + 4*p + i] = value of row 4*strip+i.
+int cute_quad_build_strips(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
+                           cute_quad_lists *out)
+{
+    if (!out || !rowPtr || (rowPtr[M] && (!cols || !vals))) return CUTE_ERR_ARG;
+    std::memset(out, 0, sizeof(*out));
+    const uint32_t S = (M + 3) / 4;
+    out->M = M;
+    out->K = K;
+    out->numRowPanels = S;
+    out->rowsPerList = 4;
+    out->groupPtr = cute::alloc_array<uint32_t>(uint64_t(S) + 1);
+    out->tail = cute::alloc_array<uint32_t>(S);
+    if (!out->groupPtr || !out->tail) { cute_quad_release(out); return CUTE_ERR_NOMEM; }
+    cute::parallel_ranges(S, 256, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            const uint32_t len = merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * 4, [](uint32_t, const float *) {});
+            out->groupPtr[q + 1] = (len + 15) / 16;
+            out->tail[q] = len ? len - 16u * ((len + 15) / 16 - 1) : 0u;
+        }
+    });
+    uint64_t total = 0, pairs = 0;
+    for (uint32_t q = 0; q < S; ++q) {
+        const uint32_t groups = out->groupPtr[q + 1];
+        pairs += groups ? uint64_t(groups - 1) * 16 + out->tail[q] : 0;
+        total += groups;
+        if (total > 0xffffffffull / 64) { cute_quad_release(out); return CUTE_ERR_SHAPE; }
+        out->groupPtr[q + 1] = uint32_t(total);
+    }
+    out->numGroups = total;
+    out->numPairs = pairs;
+    out->cols = cute::alloc_array<uint32_t>(total * 16);
+    out->vals = cute::alloc_array<float>(total * 64);
+    if (!out->cols || !out->vals) { cute_quad_release(out); return CUTE_ERR_NOMEM; }
+    cute::parallel_ranges(S, 256, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            const uint64_t g0 = out->groupPtr[q];
+            const uint32_t slots = (out->groupPtr[q + 1] - out->groupPtr[q]) * 16;
+            uint32_t s = 0, last = 0;
+            merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * 4, [&](uint32_t col, const float *v) {
+                out->cols[g0 * 16 + s] = col;
+                std::memcpy(out->vals + g0 * 64 + 4 * uint64_t(s), v, 4 * sizeof(float));
+                last = col;
+                ++s;
+            });
+            for (; s < slots; ++s) out->cols[g0 * 16 + s] = last;
         }
     });
     return CUTE_OK;

@@ -407,7 +407,9 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
 // each, a contiguous 256-byte piece of a B row.  Two operand sets roll: as soon as the MFMA of
 // pair p is issued, B operand p of the group after next is requested into the same register.
 //
-// chunks[i] = {first group, end group, row panel, atomic}; launch: x walks the chunks, y the slabs.
+// chunks[i] = {first group, end group, row panel (or 4-row strip), atomic}; launch: x walks
+// the chunks, y the slabs.  STRIPS: one list per 4-row strip (cute_quad_build_strips) instead of four
+// lockstep lists per panel; the instruction stream is the same, only the accumulators mean something else.
 // Addresses are 32-bit byte offsets from scalar bases; the planner checks the sizes.
 // ---------------------------------------------------------------------------------------
 template <int P>
@@ -421,7 +423,7 @@ __device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32
     return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(B) + (__umul24(col, row_pitch) + col_off));
 }
 
-template <bool FULL>
+template <bool FULL, bool STRIPS>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
     const float *__restrict__ qvals, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
@@ -513,16 +515,30 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
 #undef CUTE_QUAD_MFMA16
     }
     if (live) {
-        uint32_t off = __umul24(panel * 16u, row_pitch) + n * 4u;
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg)
+        if (STRIPS) {
+            // all 16 pairs of a group belong to one 4-row strip; the four accumulators only break
+            // the dependency chain and are summed here
+            const f32x4 sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+            uint32_t off = __umul24(panel * 4u, row_pitch) + n * 4u;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                if (atomic) unsafeAtomicAdd(dst, acc[rg][i]);
-                else __builtin_nontemporal_store(acc[rg][i], dst);   // C is not read again: keep it out of the L2
+                if (atomic) unsafeAtomicAdd(dst, sum[i]);
+                else __builtin_nontemporal_store(sum[i], dst);
                 off += row_pitch;
             }
+        } else {
+            uint32_t off = __umul24(panel * 16u, row_pitch) + n * 4u;
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
+                    if (atomic) unsafeAtomicAdd(dst, acc[rg][i]);
+                    else __builtin_nontemporal_store(acc[rg][i], dst);   // C is not read again: keep it out of the L2
+                    off += row_pitch;
+                }
+        }
     }
 }
 
@@ -589,13 +605,14 @@ __global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict
     }
 }
 
-// Zero the C rows of the listed 16-row panels (those whose chunks combine through atomics).
-__global__ void zero_panels(const uint32_t *__restrict__ panels, uint32_t count, float *__restrict__ C, uint32_t N)
+// Zero the C rows of the listed panels (16 rows) or strips (4 rows): those whose chunks combine through atomics.
+__global__ void zero_panels(const uint32_t *__restrict__ panels, uint32_t count, uint32_t rows_per_panel,
+                            float *__restrict__ C, uint32_t N)
 {
     const uint32_t p = blockIdx.x;
     if (p >= count) return;
-    float *base = C + size_t(panels[p]) * 16u * N;
-    for (uint32_t i = threadIdx.x; i < 16u * N; i += blockDim.x) base[i] = 0.0f;
+    float *base = C + size_t(panels[p]) * rows_per_panel * N;
+    for (uint32_t i = threadIdx.x; i < rows_per_panel * N; i += blockDim.x) base[i] = 0.0f;
 }
 
 // One group of L = 1<<LOG_L lanes per row; lane t of the group owns VEC consecutive columns

@@ -143,15 +143,23 @@ void cute_hrpb_tiled_release(cute_hrpb_tiled *t);
  * column of their list (column 0 for an empty list) with zero values.
  * ---------------------------------------------------------------------------------- */
 typedef struct cute_quad_lists {
-    uint32_t M, K, numRowPanels;
+    uint32_t M, K, numRowPanels;   /* numRowPanels: number of list units (16-row panels, or 4-row strips)  */
     uint64_t numGroups;
     uint32_t *groupPtr;        /* [numRowPanels+1]                                         */
     uint32_t *cols;            /* [numGroups*16]                                           */
     float *vals;               /* [numGroups*64]                                           */
+    uint32_t *tail;            /* [numRowPanels] pair slots in use in the unit's last group (0 if it has none) */
+    uint64_t numPairs;         /* (row group, column) pairs that hold a nonzero            */
+    uint32_t rowsPerList;      /* 16: four lockstep lists per panel; 4: one list per strip */
 } cute_quad_lists;
 
 int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
                     cute_quad_lists *out);
+/* One list per 4-row strip (numRowPanels = M/4), nothing padded to a neighbour: for matrices with a
+ * few very long rows.  A group is 16 consecutive pairs of one strip: cols[g*16 + p],
+ * vals[g*64 + 4*p + i] = value of row 4*strip+i. */
+int cute_quad_build_strips(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
+                           cute_quad_lists *out);
 void cute_quad_release(cute_quad_lists *q);
 
 /* ------------------------------------------------------------------------------------
@@ -275,6 +283,9 @@ float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, cons
  * ---------------------------------------------------------------------------------- */
 typedef struct cute_hrpb_dev cute_hrpb_dev;
 int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out);
+/* Same, with the quad-list layout forced: 0 library's choice (lockstep lists unless they would be less
+ * than 60 % full), 1 four lockstep lists per 16-row panel, 2 one list per 4-row strip. */
+int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_dev **out);
 void cute_hrpb_dev_free(cute_hrpb_dev *d);
 uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d); /* device bytes held */
 

@@ -340,3 +340,32 @@ def test_full_size_other_configs(cs, orc, torch_cuda, cfg):
     bound = scale @ np.abs(B.astype(np.float64))
     got = out.sum(0, dtype=np.float64)
     assert (np.abs(got - expect) <= 1e-5 * bound).all()
+
+
+def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
+    """The quad kernel on one list per 4-row strip (forced, and chosen by the library for a matrix
+    with a few very long rows), including split strips that combine through atomics."""
+    torch = torch_cuda
+    rng = np.random.default_rng(21)
+    M, K = 512, 4096
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 2500 if r in (7, 130, 131) else 3)
+    for N in (64, 100):
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        dB = torch.from_numpy(B).cuda()
+        for layout, kw in ((2, {}), (2, dict(max_chunk_blocks=3)), (0, {}), (1, {})):
+            h = cs.HRPB(M, K, rp, cl, vl)
+            h.upload(quad_layout=layout)
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            plan = cs.SPMM_TC(h, N, path=cs.PATH_BRICK, mfma_shape=2, **kw)
+            plan.run(dB, dC)
+            plan.run(dB, dC)                        # a second launch must not add onto the first
+            torch.cuda.synchronize()
+            assert cs.backward_error(rp, cl, vl, B, ref, dC.cpu().numpy()) <= BERR, (N, layout, kw, plan.info)
+    # integer inputs: bit for bit, strips forced on an ordinary matrix
+    rp, cl, vl = random_csr(rng, 256, 320, density=0.05, values="ints")
+    B = rng.integers(-4, 5, (320, 96)).astype(np.float32)
+    h = cs.HRPB(256, 320, rp, cl, vl)
+    h.upload(quad_layout=2)
+    out, _ = _run(cs, torch, h, B, path=cs.PATH_BRICK, mfma_shape=2)
+    assert (out == orc.spmm_csr(rp, cl, vl, B)).all()

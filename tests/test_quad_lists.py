@@ -80,3 +80,46 @@ def test_quad_build_rejects_null_arguments(cs):
     import ctypes as C
     lib = cs.load_library()
     assert lib.cute_quad_build(16, 16, None, None, None, None) == -5
+
+
+@pytest.mark.parametrize("name,case", list(_cases()), ids=[n for n, _ in _cases()])
+def test_strip_lists_hold_exactly_the_matrix(cs, name, case):
+    """One list per 4-row strip: same content, no padding beyond a strip's own last group."""
+    M, K, rp, cl, vl = case
+    q = cs.quad_lists(M, K, rp, cl, vl, strips=True)
+    gp = q["groupPtr"].astype(np.int64)
+    assert q["rowsPerList"] == 4 and len(gp) == M // 4 + 1 and gp[-1] == q["numGroups"]
+    entries, pairs = {}, 0
+    for st in range(M // 4):
+        rows = range(4 * st, 4 * st + 4)
+        want = sorted({int(c) for r in rows for c in cl[rp[r]:rp[r + 1]]})
+        pairs += len(want)
+        assert gp[st + 1] - gp[st] == (len(want) + 15) // 16, (name, st)
+        assert q["tail"][st] == (len(want) - 16 * ((len(want) + 15) // 16 - 1) if want else 0)
+        slots = [int(c) for g in range(gp[st], gp[st + 1]) for c in q["cols"][g]]
+        assert slots[:len(want)] == want and all(c == want[-1] for c in slots[len(want):])
+        for g in range(gp[st], gp[st + 1]):
+            for p in range(16):
+                for i in range(4):
+                    v = q["vals"][g, 4 * p + i]
+                    if v != 0:
+                        assert (16 * (g - gp[st]) + p) < len(want)
+                        entries[(4 * st + i, int(q["cols"][g, p]))] = v
+    expect = {(r, int(cl[k])): vl[k] for r in range(M) for k in range(rp[r], rp[r + 1]) if vl[k] != 0}
+    assert entries.keys() == expect.keys() and q["numPairs"] == pairs
+    assert all(np.float32(entries[k]).tobytes() == np.float32(expect[k]).tobytes() for k in expect)
+
+
+def test_lockstep_tail_and_pair_count(cs):
+    rng = np.random.default_rng(2)
+    M, K = 64, 128
+    rp, cl, vl = random_csr(rng, M, K, density=0.07)
+    q = cs.quad_lists(M, K, rp, cl, vl)
+    gp = q["groupPtr"].astype(np.int64)
+    pairs = 0
+    for p in range(M // 16):
+        lens = [len({int(c) for r in range(16 * p + 4 * rg, 16 * p + 4 * rg + 4) for c in cl[rp[r]:rp[r + 1]]}) for rg in range(4)]
+        pairs += sum(lens)
+        L = max(lens)
+        assert q["tail"][p] == (4 * (L - 4 * ((L + 3) // 4 - 1)) if L else 0)
+    assert q["numPairs"] == pairs and q["rowsPerList"] == 16
