@@ -353,7 +353,7 @@ def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
         B = rng.standard_normal((K, N)).astype(np.float32)
         ref = orc.spmm_csr(rp, cl, vl, B)
         dB = torch.from_numpy(B).cuda()
-        for layout, kw in ((2, {}), (2, dict(max_chunk_blocks=3)), (0, {}), (1, {})):
+        for layout, kw in ((2, {}), (2, dict(max_chunk_blocks=3)), (2, dict(slots=64)), (0, {}), (1, {})):
             h = cs.HRPB(M, K, rp, cl, vl)
             h.upload(quad_layout=layout)
             dC = torch.full((M, N), float("nan"), device="cuda")
