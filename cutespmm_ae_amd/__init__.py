@@ -21,7 +21,7 @@ ABI_SYMBOLS = [
     "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
-    "cute_quad_build", "cute_quad_build_strips", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
+    "cute_quad_build", "cute_quad_fill", "cute_quad_build_strips", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",

@@ -193,12 +193,14 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
         // Lockstep lists unless they would be mostly padding (a few very long rows stretch the
         // lists of their neighbours): then one list per 4-row strip.
         cute_quad_lists ql;
-        rc = quad_layout == 2 ? cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql)
-                              : cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
-        if (rc == CUTE_OK && quad_layout == 0 && ql.numGroups && double(ql.numPairs) < 0.6 * 16.0 * double(ql.numGroups)) {
-            cute_quad_release(&ql);
-            rc = cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
+        if (quad_layout == 0) {
+            uint64_t groups = 0, pairs = 0;
+            rc = cute_quad_fill(h->M, h->rowPtr, h->cols, &groups, &pairs);
+            quad_layout = (groups && double(pairs) < 0.6 * 16.0 * double(groups)) ? 2 : 1;
         }
+        if (rc == CUTE_OK)
+            rc = quad_layout == 2 ? cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql)
+                                  : cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
         if (rc == CUTE_OK) {
             d->numGroups = ql.numGroups;
             d->quadRows = ql.rowsPerList;

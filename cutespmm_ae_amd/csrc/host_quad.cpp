@@ -62,6 +62,29 @@ void cute_quad_release(cute_quad_lists *q)
     std::memset(q, 0, sizeof(*q));
 }
 
+int cute_quad_fill(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, uint64_t *numGroups, uint64_t *numPairs)
+{
+    if (!rowPtr || !numGroups || !numPairs || (rowPtr[M] && !cols)) return CUTE_ERR_ARG;
+    const uint32_t P = (M + CUTE_TM - 1) / CUTE_TM;
+    std::vector<uint64_t> groups_of(P, 0), pairs_of(P, 0);
+    cute::parallel_ranges(P, 64, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            uint32_t longest = 0;
+            for (uint32_t rg = 0; rg < 4; ++rg) {
+                // values are not looked at: any non-null array of the right length does
+                const uint32_t len = merge_row_group(M, rowPtr, cols, reinterpret_cast<const float *>(cols),
+                                                     uint32_t(q) * CUTE_TM + rg * 4, [](uint32_t, const float *) {});
+                longest = std::max(longest, len);
+                pairs_of[q] += len;
+            }
+            groups_of[q] = (longest + 3) / 4;
+        }
+    });
+    *numGroups = *numPairs = 0;
+    for (uint32_t q = 0; q < P; ++q) { *numGroups += groups_of[q]; *numPairs += pairs_of[q]; }
+    return CUTE_OK;
+}
+
 int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
                     cute_quad_lists *out)
 {

@@ -155,6 +155,9 @@ typedef struct cute_quad_lists {
 
 int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
                     cute_quad_lists *out);
+/* Size of the lockstep layout without building it: its groups and its occupied pairs (fill =
+ * numPairs / (16 * numGroups)); cute_hrpb_upload uses it to choose between the two layouts. */
+int cute_quad_fill(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, uint64_t *numGroups, uint64_t *numPairs);
 /* One list per 4-row strip (numRowPanels = M/4), nothing padded to a neighbour: for matrices with a
  * few very long rows.  A group is 16 consecutive pairs of one strip: cols[g*16 + p],
  * vals[g*64 + 4*p + i] = value of row 4*strip+i. */

@@ -123,3 +123,9 @@ def test_lockstep_tail_and_pair_count(cs):
         L = max(lens)
         assert q["tail"][p] == (4 * (L - 4 * ((L + 3) // 4 - 1)) if L else 0)
     assert q["numPairs"] == pairs and q["rowsPerList"] == 16
+    import ctypes as C
+    g, n = C.c_uint64(), C.c_uint64()
+    rp32, cl32 = np.ascontiguousarray(rp, np.uint32), np.ascontiguousarray(cl, np.uint32)
+    assert cs.load_library().cute_quad_fill(M, rp32.ctypes.data_as(C.POINTER(C.c_uint32)), cl32.ctypes.data_as(C.POINTER(C.c_uint32)),
+                                            C.byref(g), C.byref(n)) == 0
+    assert (g.value, n.value) == (q["numGroups"], pairs)
