@@ -128,7 +128,7 @@ def main():
         kernels.append("zero_panels")
     if plan.info["numChunks"]:
         kernels.append(plan.kernel_name)
-    if plan.info["numRowPanelsSparse"] or plan.info["numEmptyPanels"]:
+    if (plan.info["numRowPanelsSparse"] or plan.info["numEmptyPanels"]) and not plan.info["fusedLaunch"]:
         kernels.append("csr_rows_batched")
     roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                     traffic=recorded_traffic(cfg["name"]), kernel=plan.kernel_name if plan.info["numChunks"] else "csr_rows_batched",

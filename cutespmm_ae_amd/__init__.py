@@ -83,7 +83,7 @@ class cute_plan_info(C.Structure):
                 ("numAtomicChunks", C.c_uint32), ("numBrickPanels", C.c_uint32), ("numRowPanelsSparse", C.c_uint32),
                 ("numEmptyPanels", C.c_uint32), ("slots", C.c_uint32), ("precision", C.c_uint32),
                 ("path", C.c_uint32), ("mfmaShape", C.c_uint32), ("pipeline", C.c_uint32),
-                ("reserved", C.c_uint32 * 3)]
+                ("fusedLaunch", C.c_uint32), ("reserved", C.c_uint32 * 2)]
 
 
 i32p = C.POINTER(C.c_int32)
@@ -530,7 +530,7 @@ class SPMM_TC:
         _check(load_library().cute_spmm_plan_info(self._plan, C.byref(info)), "cute_spmm_plan_info")
         self.info = {k: getattr(info, k) for k, _ in cute_plan_info._fields_ if k != "reserved"}
         self.numRowPanelsSplit = info.numChunks
-        self.kernel_name = ("hrpb_quad_f32" if info.mfmaShape == 2 else
+        self.kernel_name = ("hrpb_quad_rows_f32" if info.fusedLaunch else "hrpb_quad_f32" if info.mfmaShape == 2 else
                             "hrpb_brick_f32_rolling" if info.pipeline == 1 else "hrpb_brick_f32")
 
     def _check_shapes(self, MatB, MatC):

@@ -407,6 +407,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->info.path = uint32_t(t.path);
     p->info.mfmaShape = uint32_t(p->shape);
     p->info.pipeline = uint32_t(p->pipeline);
+    p->info.fusedLaunch = (p->shape == 2 && !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 4) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
 }
@@ -565,6 +566,28 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
         const bool full = N % 64u == 0, strips = p->d->quadRows == 4;
+        // mixed plan: quad chunks and sparse rows in one launch (instantiated for 4-float lanes and 16..64 lanes per row)
+        const uint64_t row_lanes = (uint64_t(p->numRows) * p->rows_slabs) << p->rows_logl;
+        const uint64_t row_blocks = (row_lanes + 255) / 256, quad_blocks = uint64_t(grid.x) * grid.y;
+        if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
+#define CUTE_FUSED_LAUNCH(F, S, LL)                                                                                       \
+    hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
+                       grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQCols, p->d->dQVals,  \
+                       p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
+#define CUTE_FUSED_LL(F, S)                                                     \
+    switch (p->rows_logl) {                                                     \
+        case 4: CUTE_FUSED_LAUNCH(F, S, 4); break;                              \
+        case 5: CUTE_FUSED_LAUNCH(F, S, 5); break;                              \
+        default: CUTE_FUSED_LAUNCH(F, S, 6); break;                             \
+    }
+            if (full && strips) { CUTE_FUSED_LL(true, true) }
+            else if (full) { CUTE_FUSED_LL(true, false) }
+            else if (strips) { CUTE_FUSED_LL(false, true) }
+            else { CUTE_FUSED_LL(false, false) }
+#undef CUTE_FUSED_LL
+#undef CUTE_FUSED_LAUNCH
+            return check_launch("spmm launch");
+        }
 #define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,        \
                        p->d->dQCols, p->d->dQVals, dB, dC, N)

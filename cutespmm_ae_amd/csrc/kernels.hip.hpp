@@ -424,13 +424,14 @@ __device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32
 }
 
 template <bool FULL, bool STRIPS>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
-    const float *__restrict__ qvals, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+__device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint4 *__restrict__ chunks,
+                                          uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
+                                          const float *__restrict__ qvals, const float *__restrict__ B,
+                                          float *__restrict__ C, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t chunk = xcd_contiguous_id(blockIdx.x, groups_per_xcd) * kWavesPerGroup + wave;
+    const uint32_t chunk = xcd_contiguous_id(block_x, groups_per_xcd) * kWavesPerGroup + wave;
     if (chunk >= num_chunks) return;
     const uint4 ck = chunks[chunk];
     const uint32_t g_end = __builtin_amdgcn_readfirstlane(ck.y);
@@ -438,7 +439,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
     const uint32_t atomic = __builtin_amdgcn_readfirstlane(ck.w);
     uint32_t g = __builtin_amdgcn_readfirstlane(ck.x);
 
-    const uint32_t n = blockIdx.y * kWaveSize + lane;
+    const uint32_t n = block_y * kWaveSize + lane;
     const bool live = FULL || n < N;
     const uint32_t row_pitch = N * 4u;
     const uint32_t col_off = (live ? n : N - 1u) * 4u;      // dead lanes re-read the last column and store nothing
@@ -540,6 +541,14 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
                 }
         }
     }
+}
+
+template <bool FULL, bool STRIPS>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
+    const float *__restrict__ qvals, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+{
+    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qcols, qvals, B, C, N);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -661,17 +670,16 @@ __global__ __launch_bounds__(256) void csr_rows(const uint32_t *__restrict__ row
 // row costs about one memory round trip per batch instead of one per nonzero.  Each C
 // element still accumulates its row in storage order.
 template <int VEC, int LOG_L, int BATCH>
-__global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restrict__ row_list, uint32_t num_rows,
-                                                        uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
-                                                        const uint32_t *__restrict__ cols,
-                                                        const float *__restrict__ vals, const float *__restrict__ B,
-                                                        float *__restrict__ C, uint32_t N)
+__device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint32_t *__restrict__ row_list, uint32_t num_rows,
+                                                  uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+                                                  const uint32_t *__restrict__ cols, const float *__restrict__ vals,
+                                                  const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
     typedef typename Vec<VEC>::type V;
     constexpr uint32_t L = 1u << LOG_L;
     constexpr uint32_t STEP = BATCH < int(L) ? uint32_t(BATCH) : L;
     const uint32_t t = threadIdx.x & (L - 1);
-    const uint64_t gid = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> LOG_L;
+    const uint64_t gid = (uint64_t(block_id) * blockDim.x + threadIdx.x) >> LOG_L;
     if (gid >= uint64_t(num_rows) * num_slabs) return;
     const uint32_t ridx = uint32_t(gid / num_slabs);
     const uint32_t slab = uint32_t(gid % num_slabs);
@@ -703,6 +711,36 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
         }
     }
     if (live) __builtin_nontemporal_store(acc, reinterpret_cast<V *>(C + size_t(row) * N + c0));
+}
+
+template <int VEC, int LOG_L, int BATCH>
+__global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restrict__ row_list, uint32_t num_rows,
+                                                        uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+                                                        const uint32_t *__restrict__ cols,
+                                                        const float *__restrict__ vals, const float *__restrict__ B,
+                                                        float *__restrict__ C, uint32_t N)
+{
+    rows_batched_body<VEC, LOG_L, BATCH>(blockIdx.x, row_list, num_rows, num_slabs, rowPtr, cols, vals, B, C, N);
+}
+
+// One launch for a plan that uses both the quad kernel and the row kernel: they write disjoint
+// panels, and the row kernel's short, even work fills the SIMDs that the quad kernel's long chunks
+// leave idle.  Blocks [0, quad_blocks) are the quad kernel's 2-D grid flattened (x fastest, so the
+// XCD of a block is still x % 8); the rest are the row kernel's blocks.
+template <bool FULL, bool STRIPS, int LOG_L>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
+    uint32_t quad_blocks_x, uint32_t quad_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
+    uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols, const float *__restrict__ qvals,
+    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, const uint32_t *__restrict__ rowPtr,
+    const uint32_t *__restrict__ cols, const float *__restrict__ vals, const float *__restrict__ B, float *__restrict__ C,
+    uint32_t N)
+{
+    static_assert(kWaveSize * kWavesPerGroup == 256, "both bodies are written for 256-thread blocks");
+    if (blockIdx.x < quad_blocks)
+        quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, chunks, num_chunks, groups_per_xcd,
+                                qcols, qvals, B, C, N);
+    else
+        rows_batched_body<4, LOG_L, 8>(blockIdx.x - quad_blocks, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
 }
 
 // Thread per C element (inc/SPMM.cuh:898-920 restated for fp32 and a 64x4 thread tile).

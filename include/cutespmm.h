@@ -331,7 +331,8 @@ typedef struct cute_plan_info {
     uint32_t precision, path;
     uint32_t mfmaShape;        /* MFMA kernel in use: 1 16x16x4 bricks, 2 4x4x1 quad lists */
     uint32_t pipeline;         /* brick kernel variant in use: 1 rolling, 2 pipelined     */
-    uint32_t reserved[3];
+    uint32_t fusedLaunch;      /* 1: quad chunks and sparse rows go out as one launch     */
+    uint32_t reserved[2];
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;
