@@ -442,7 +442,9 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
                      const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
 {
     const uint64_t lanes = (uint64_t(num_rows) * slabs) << logl;
-    const dim3 grid(uint32_t((lanes + 255) / 256)), block(256);
+    // the batched kernel remaps its blocks per XCD and wants a multiple of 8 of them
+    const uint32_t blocks = uint32_t((lanes + 255) / 256);
+    const dim3 grid(BATCHED ? (blocks + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd : blocks), block(256);
 #define CUTE_ROWS_CASE(LL)                                                                                        \
     case LL:                                                                                                      \
         if (BATCHED)                                                                                              \

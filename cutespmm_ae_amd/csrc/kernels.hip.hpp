@@ -720,7 +720,10 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
                                                         const float *__restrict__ vals, const float *__restrict__ B,
                                                         float *__restrict__ C, uint32_t N)
 {
-    rows_batched_body<VEC, LOG_L, BATCH>(blockIdx.x, row_list, num_rows, num_slabs, rowPtr, cols, vals, B, C, N);
+    // the grid is a multiple of the XCD count: each XCD walks one contiguous range of rows, so the B rows
+    // that neighbouring rows share stay in that XCD's L2
+    rows_batched_body<VEC, LOG_L, BATCH>(xcd_contiguous_id(blockIdx.x, gridDim.x / kNumXcd), row_list, num_rows, num_slabs,
+                                         rowPtr, cols, vals, B, C, N);
 }
 
 // One launch for a plan that uses both the quad kernel and the row kernel: they write disjoint
