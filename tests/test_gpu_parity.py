@@ -369,3 +369,40 @@ def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
     h.upload(quad_layout=2)
     out, _ = _run(cs, torch, h, B, path=cs.PATH_BRICK, mfma_shape=2)
     assert (out == orc.spmm_csr(rp, cl, vl, B)).all()
+
+
+def test_launches_can_be_captured_in_a_graph(cs, orc, torch_cuda):
+    """cute_spmm_run only enqueues kernels (zeroing included), so a caller may capture it in a HIP
+    graph: every replay, with B changed in place between replays, equals the eager result."""
+    torch = torch_cuda
+    rng = np.random.default_rng(9)
+    M, K, N = 512, 4096, 128
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1200 if r in (5, 300) else 6)     # split panels: atomics + zeroing
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for kw in (dict(), dict(path=cs.PATH_BRICK, mfma_shape=1), dict(path=cs.PATH_BRICK, mfma_shape=2)):
+        plan = cs.SPMM_TC(h, N, **kw)
+        dB = torch.zeros((K, N), device="cuda")
+        dC = torch.full((M, N), float("nan"), device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            plan.run(dB, dC, stream=side)                   # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(dB, dC, stream=torch.cuda.current_stream())
+        for rep in range(3):
+            B = rng.standard_normal((K, N)).astype(np.float32)
+            dB.copy_(torch.from_numpy(B))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = dC.cpu().numpy()
+            eager = torch.full((M, N), float("nan"), device="cuda")
+            plan.run(dB, eager)
+            torch.cuda.synchronize()
+            ref = orc.spmm_csr(rp, cl, vl, B)
+            assert cs.backward_error(rp, cl, vl, B, ref, got) <= BERR, (kw, rep)
+            if not plan.info["numAtomicChunks"]:
+                assert (got == eager.cpu().numpy()).all(), (kw, rep)
