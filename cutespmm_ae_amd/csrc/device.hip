@@ -539,7 +539,9 @@ template <int VEC, bool ACC>
 void launch_blocked_ell(const cute_blocked_ell_dev *d, const float *dB, float *dC, uint32_t N, hipStream_t s)
 {
     const uint32_t rows = uint32_t(d->height) * uint32_t(d->blockSize), strips = rows / 16u;
-    const dim3 grid((strips + 3u) / 4u, (N + 16u * VEC - 1u) / (16u * VEC)), block(256);
+    // x extent a multiple of the XCD count: the kernel maps x so that each XCD owns a contiguous range of strips
+    const uint32_t groups = (((strips + 3u) / 4u + 7u) / 8u) * 8u;
+    const dim3 grid(groups, (N + 16u * VEC - 1u) / (16u * VEC)), block(256);
     if (N % (16u * VEC) == 0)
         hipLaunchKernelGGL((cute_dev::blocked_ell_f32<VEC, true, ACC>), grid, block, 0, s, d->dColIdx, d->dValues,
                            uint32_t(d->blockSize), uint32_t(d->width), strips, rows, dB, dC, N);

@@ -562,6 +562,8 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
 // lane VEC consecutive C columns are those of the brick kernel.
 // ACCUMULATE: C += A.B (for the heavy part of a split matrix), else C = A.B.
 // ---------------------------------------------------------------------------------------
+constexpr int kEllDepth = 3;
+
 template <int VEC, bool FULL, bool ACCUMULATE>
 __global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict__ ell_col, const float *__restrict__ ell_val,
                                                        uint32_t block_size, uint32_t width, uint32_t num_strips,
@@ -570,35 +572,75 @@ __global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict
 {
     typedef typename Vec<VEC>::type V;
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const uint32_t strip = blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+    // neighbouring strips reference neighbouring block columns: keep them on one XCD, whose L2 then holds
+    // their B rows (gridDim.x is a multiple of the XCD count)
+    const uint32_t strip = xcd_contiguous_id(blockIdx.x, gridDim.x / kNumXcd) * (blockDim.x / kWaveSize) +
+                           __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
     if (strip >= num_strips) return;
     const uint32_t row16 = lane & 15u, q = lane >> 4;
     const uint32_t c0 = blockIdx.y * (16u * VEC) + row16 * VEC;       // this lane's VEC columns of the slab
     const bool col_live = FULL || c0 < N;
     const uint32_t block_row = (strip * 16u) / block_size;
+    const uint32_t tiles_per_block = block_size / 16u;                // 16-wide k tiles of one block
     const size_t pitch = size_t(width) * block_size;
     const float *a_row = ell_val + size_t(strip * 16u + row16) * pitch + q * 4u;
     const int32_t *cols = ell_col + size_t(block_row) * width;
+    const float *b_base = B + size_t(q * 4u) * N + (col_live ? c0 : 0u);
 
     f32x4 acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = f32x4(0.0f);
 
-    for (uint32_t w = 0; w < width; ++w) {
-        const int32_t bc = cols[w];
-        if (bc < 0) break;                                            // padding follows the last block
-        for (uint32_t kt = 0; kt < block_size; kt += 16u) {           // 16-wide k tiles of the block
-            const f32x4 a = *reinterpret_cast<const f32x4 *>(a_row + size_t(w) * block_size + kt);
-            const float *b_row = B + size_t(uint32_t(bc) * block_size + kt + q * 4u) * N + c0;
-            V b[4];
+    struct Operands {
+        f32x4 a;
+        V b[4];
+        bool past;                    // wave-uniform: the set holds a re-read of the last tile and must not count
+    };
+    // Block ids are taken 64 at a time into one vector register (lane i holds block w0 + i);
+    // the padding (-1) that follows the last block ends the row.  Inside such a batch the k
+    // tiles roll through kEllDepth operand sets: a set is refilled with tile t+kEllDepth right
+    // after the MFMAs of tile t, and the id of a tile's block comes out of the register by readlane, so no load
+    // depends on another load.
+    for (uint32_t w0 = 0; w0 < width; w0 += kWaveSize) {
+        const uint32_t in_batch = min(width - w0, uint32_t(kWaveSize));
+        const int32_t ids = lane < in_batch ? cols[w0 + lane] : -1;
+        const uint64_t pad = __ballot(ids < 0);
+        const uint32_t valid = pad ? uint32_t(__builtin_ctzll(pad)) : uint32_t(kWaveSize);
+        const uint32_t tiles = valid * tiles_per_block;
+        if (tiles == 0) break;
+        auto fetch = [&](uint32_t t, Operands &o) {
+            o.past = t >= tiles;                                      // past the end: re-read the last tile
+            t = min(t, tiles - 1u);
+            const uint32_t w = t / tiles_per_block, kt = (t % tiles_per_block) * 16u;
+            const uint32_t bc = uint32_t(__builtin_amdgcn_readlane(ids, w));
+            o.a = *reinterpret_cast<const f32x4 *>(a_row + size_t(w0 + w) * block_size + kt);
+            const float *b_row = b_base + size_t(bc * block_size + kt) * N;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) b[e] = col_live ? *reinterpret_cast<const V *>(b_row + size_t(e) * N) : V(0.0f);
+            for (int e = 0; e < 4; ++e) o.b[e] = *reinterpret_cast<const V *>(b_row + size_t(e) * N);
+        };
+        auto multiply = [&](const Operands &o) {
+            const f32x4 a = o.past ? f32x4(0.0f) : o.a;               // masked here, where the data is waited for anyway
 #pragma unroll
             for (int e = 0; e < 4; ++e)
 #pragma unroll
                 for (int v = 0; v < VEC; ++v)
-                    acc[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], vec_get<VEC>(b[e], v), acc[v], 0, 0, 0);
+                    acc[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], vec_get<VEC>(o.b[e], v), acc[v], 0, 0, 0);
+        };
+        Operands o[kEllDepth];
+#pragma unroll
+        for (int k = 0; k < kEllDepth; ++k) fetch(uint32_t(k), o[k]);
+        __builtin_amdgcn_sched_barrier(0);
+        for (uint32_t t = 0; t < tiles; t += kEllDepth) {
+#pragma unroll
+            for (int k = 0; k < kEllDepth; ++k) {
+                // the fences keep the compiler from sinking the loads to their first use
+                multiply(o[k]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(t + uint32_t(k) + kEllDepth, o[k]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
+        if (valid < in_batch) break;
     }
     if (!col_live) return;
     const uint32_t r0 = strip * 16u + q * 4u;
