@@ -90,15 +90,18 @@ def partition(blockedRowPtr, nbN, slots):
     return out[:n].copy()
 
 
-def spmm_coo(rows, cols, vals, B, M):
+def spmm_coo(rows, cols, vals, B, M, inner_parallel=False):
+    """inc.h:71-83.  inner_parallel=True keeps the reference's placement of the parallel loop
+    (inside the loop over nonzeros); the result is the same, bit for bit."""
     rows = np.ascontiguousarray(rows, np.uint32)
     cols = np.ascontiguousarray(cols, np.uint32)
     vals = np.ascontiguousarray(vals, np.float32)
     B = np.ascontiguousarray(B, np.float32)
     K, N = B.shape
     Cm = np.empty((M, N), np.float32)
-    lib().orc_spmm_coo(_p(rows, C.c_uint32), _p(cols, C.c_uint32), _p(vals, C.c_float), _p(B, C.c_float),
-                       _p(Cm, C.c_float), C.c_uint32(M), C.c_uint32(K), C.c_uint32(N), C.c_uint32(len(vals)))
+    fn = lib().orc_spmm_coo_inner_parallel if inner_parallel else lib().orc_spmm_coo
+    fn(_p(rows, C.c_uint32), _p(cols, C.c_uint32), _p(vals, C.c_float), _p(B, C.c_float),
+       _p(Cm, C.c_float), C.c_uint32(M), C.c_uint32(K), C.c_uint32(N), C.c_uint32(len(vals)))
     return Cm
 
 

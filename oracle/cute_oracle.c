@@ -329,6 +329,24 @@ void orc_spmm_coo(const uint32_t *rows, const uint32_t *cols, const float *vals,
     }
 }
 
+/* The loop structure of inc.h:71-83 as written there: the nonzeros are walked serially and
+ * the thread team is forked and joined inside, once per nonzero, over the N columns.  Same
+ * sums in the same order as orc_spmm_coo; kept to show what that structure costs (one
+ * fork/join per nonzero), which is why the timed CPU baseline is the row-parallel form. */
+void orc_spmm_coo_inner_parallel(const uint32_t *rows, const uint32_t *cols, const float *vals, const float *B,
+                                 float *C, uint32_t M, uint32_t K, uint32_t N, uint32_t nnz)
+{
+    (void)K;
+    memset(C, 0, (size_t)M * N * sizeof(float));
+    for (uint32_t i = 0; i < nnz; ++i) {
+        const float *b = B + (size_t)cols[i] * N;
+        float *c = C + (size_t)rows[i] * N;
+        const float v = vals[i];
+#pragma omp parallel for
+        for (uint32_t j = 0; j < N; ++j) c[j] += v * b[j];
+    }
+}
+
 /* The same sums, ordered by CSR row (each C element accumulates its row's
  * nonzeros in storage order, exactly as the COO loop does for row-major COO).
  * Rows are independent, so they may be spread over threads without changing a bit. */

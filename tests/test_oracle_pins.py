@@ -200,6 +200,7 @@ def test_spmm_against_float64_dense_and_scipy(orc):
     c_coo = orc.spmm_coo(rows, cl, vl, B, M)
     c_csr = orc.spmm_csr(rp, cl, vl, B)
     assert (c_coo == c_csr).all()                       # same sums in the same order
+    assert (orc.spmm_coo(rows, cl, vl, B, M, inner_parallel=True) == c_coo).all()   # the reference's loop placement
     assert (np.abs(c_csr - exact) <= bound).all()
     s = sp.csr_matrix((vl.astype(np.float64), cl.astype(np.int64), rp.astype(np.int64)), shape=(M, K)) @ B.astype(np.float64)
     assert np.allclose(c_csr, s, rtol=1e-5, atol=1e-5)
