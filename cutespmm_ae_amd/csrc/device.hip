@@ -286,6 +286,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    p->rows_vec = p->vec;
+    // a brick work item spans 16*VEC columns: for narrow N take the narrowest tile that still covers N
+    while (p->vec > 1 && 8u * uint32_t(p->vec) >= N) p->vec /= 2;
     p->ng = (p->vec == 4 && N >= 128) ? 2 : 1;   // two column groups per lane pay off from 128 columns on (measured)
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
     if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
@@ -311,7 +314,6 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     const uint32_t num_slabs = (N + slab - 1) / slab;
     if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
     // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
-    p->rows_vec = p->vec;
     {
         uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
         while ((1u << logl) < need && logl < 6) ++logl;
@@ -346,7 +348,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             if (!to_rows[q / upp] && unit[q + 1] != unit[q]) { work += unit[q + 1] - unit[q]; ++busy; }
         const uint64_t mean = busy ? (work + busy - 1) / busy : 1;
         const uint64_t share = (work * num_slabs + resident - 1) / resident;
-        const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, mean), 8));
+        // the mean only counts while it is short: a matrix whose few MFMA panels are all very long
+        // (a handful of dense rows) must still be cut, or one wavefront walks a whole panel alone
+        const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, std::min<uint64_t>(mean, 16)), 8));
         for (uint32_t q = 0; q < num_units; ++q) {
             const uint32_t s = unit[q], e = unit[q + 1];
             if (s == e || to_rows[q / upp]) continue;
@@ -407,7 +411,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->info.path = uint32_t(t.path);
     p->info.mfmaShape = uint32_t(p->shape);
     p->info.pipeline = uint32_t(p->pipeline);
-    p->info.fusedLaunch = (p->shape == 2 && !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 4) ? 1u : 0u;
+    p->info.fusedLaunch = (p->shape == 2 && !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
 }
@@ -570,7 +574,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
         const bool full = N % 64u == 0, strips = p->d->quadRows == 4;
-        // mixed plan: quad chunks and sparse rows in one launch (instantiated for 4-float lanes and 16..64 lanes per row)
+        // mixed plan: quad chunks and sparse rows in one launch (instantiated for 4-float lanes and 4..64 lanes per row)
         const uint64_t row_lanes = (uint64_t(p->numRows) * p->rows_slabs) << p->rows_logl;
         const uint64_t row_blocks = (row_lanes + 255) / 256, quad_blocks = uint64_t(grid.x) * grid.y;
         if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
@@ -580,6 +584,8 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
                        p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
+        case 2: CUTE_FUSED_LAUNCH(F, S, 2); break;                              \
+        case 3: CUTE_FUSED_LAUNCH(F, S, 3); break;                              \
         case 4: CUTE_FUSED_LAUNCH(F, S, 4); break;                              \
         case 5: CUTE_FUSED_LAUNCH(F, S, 5); break;                              \
         default: CUTE_FUSED_LAUNCH(F, S, 6); break;                             \
