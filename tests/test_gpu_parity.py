@@ -371,6 +371,49 @@ def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
     assert (out == orc.spmm_csr(rp, cl, vl, B)).all()
 
 
+def test_mixed_plans_at_narrow_widths(cs, orc, torch_cuda):
+    """Dense panels next to sparse ones, so the planner mixes the MFMA and the row kernel: one fused
+    launch from 16 columns on (also for 4 and 8 lanes per row), narrow brick tiles for N <= 32."""
+    rng = np.random.default_rng(33)
+    M, K = 640, 2048
+    dense_rows = set(range(64, 160)) | set(range(400, 432))
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 40 if r in dense_rows else 3)
+    # the dense panels share their columns, as blocks of a stiffness matrix do
+    for r in dense_rows:
+        s, e = int(rp[r]), int(rp[r + 1])
+        cl[s:e] = np.sort(rng.choice(np.arange((r // 16) * 8, (r // 16) * 8 + 64), e - s, replace=False)).astype(cl.dtype)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for N in (4, 8, 16, 20, 24, 32, 40, 64):
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        for kw in (dict(), dict(mfma_shape=1), dict(mfma_shape=2)):
+            out, plan = _run(cs, torch_cuda, h, B, **kw)
+            info = plan.info
+            assert info["numChunks"] > 0 and info["numRowPanelsSparse"] > 0, (N, kw, info)
+            assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (N, kw, info)
+            if info["mfmaShape"] == 2:
+                assert info["fusedLaunch"] == (1 if N % 4 == 0 and N >= 16 else 0), (N, info)
+            else:
+                vec = 4 if N % 4 == 0 else 2 if N % 2 == 0 else 1
+                while vec > 1 and 8 * vec >= N:         # the narrowest tile that still covers N
+                    vec //= 2
+                assert info["slabWidth"] == 16 * vec * (2 if vec == 4 and N >= 128 else 1), (N, info)
+
+
+def test_few_huge_panels_are_still_cut(cs, orc, torch_cuda):
+    """A handful of dense rows among many short ones: only their panels go to the MFMA kernel, all of
+    them long.  Their mean length must not become the chunk length, or one wavefront walks a panel alone."""
+    rng = np.random.default_rng(34)
+    M, K, N = 4096, 8192, 32
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 6000 if r in (100, 2000, 3000) else 2)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    out, plan = _run(cs, torch_cuda, h, B)
+    assert plan.info["numBrickPanels"] == 3 and plan.info["numAtomicChunks"] >= 3 * 10, plan.info
+    assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
+
+
 def test_launches_can_be_captured_in_a_graph(cs, orc, torch_cuda):
     """cute_spmm_run only enqueues kernels (zeroing included), so a caller may capture it in a HIP
     graph: every replay, with B changed in place between replays, equals the eager result."""
