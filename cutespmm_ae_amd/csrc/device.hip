@@ -303,11 +303,16 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     else {
         // A 16x4 brick costs the same matrix time however few nonzeros it holds; the quad lists
         // only pay for occupied (4-row group, column) pairs but fetch a B row once per row group
-        // instead of once per panel.  Measured break-even: about 14 nonzeros per brick.
-        uint64_t nz = 0, bricks = 0;
+        // instead of once per panel, and pad their lists.  Measured break-even on the benchmark
+        // matrices and on the reference's 43: about 8 list slots (pairs plus padding) per brick.
+        const uint32_t lists = d->quadRows == 4 ? 4u : 1u;     // list units per panel
+        uint64_t slots = 0, bricks = 0;
         for (uint32_t q = 0; q < d->P; ++q)
-            if (!to_rows[q]) { nz += d->panelNnz[q]; bricks += (d->panelCols[q] + 3u) / 4u; }
-        p->shape = nz < 14u * bricks ? 2 : 1;
+            if (!to_rows[q]) {
+                slots += uint64_t(d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
+                bricks += (d->panelCols[q] + 3u) / 4u;
+            }
+        p->shape = slots < 8u * bricks ? 2 : 1;
     }
     if (p->shape == 2 && !(offsets_fit && d->numGroups * 64u * 4u <= 0xffffffffull)) p->shape = 1;
     const uint32_t slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
