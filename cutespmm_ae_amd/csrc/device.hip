@@ -104,6 +104,8 @@ struct cute_spmm_plan {
     uint32_t atomicPanelRows = CUTE_TM; // rows of one entry of dAtomicPanels
     uint32_t *dRowList = nullptr;
     uint32_t numRows = 0;
+    cute_dev::XcdRanges rowRanges{};   // row-kernel blocks of each XCD, balanced by nonzeros
+    uint32_t rowBlocksPerXcd = 0;       // longest of those ranges
 };
 
 extern "C" {
@@ -275,10 +277,14 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         else if (t.path == CUTE_PATH_BRICK) rows = false;
         else if (t.path == CUTE_PATH_ROWS) rows = true;
         else {
-            // Row kernel when a fetched B row serves hardly more than one nonzero of the panel
-            // (the 16-row MFMA then buys nothing) -- unless a row is so long that one lane group
+            // Row kernel when a B row fetched by the MFMA side serves hardly more than one nonzero of the
+            // panel (the matrix cores then buy nothing) -- unless a row is so long that one lane group
             // would serialise it: the brick kernel cuts long panels into balanced chunks.
-            rows = float(d->panelNnz[q]) < reuse_bar * float(d->panelCols[q]) && d->panelMaxRow[q] <= max_row_for_rows;
+            // what the MFMA side would fetch for this panel: one B row per list slot of the quad
+            // lists (pairs plus padding), which is at least one per active column
+            const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
+            const uint32_t fetches = std::max(d->panelCols[q], (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u);
+            rows = float(d->panelNnz[q]) < reuse_bar * float(fetches) && d->panelMaxRow[q] <= max_row_for_rows;
         }
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;
@@ -396,6 +402,30 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         if (to_rows[q])
             for (uint32_t r = 0; r < CUTE_TM; ++r) row_list.push_back(q * CUTE_TM + r);
 
+    // Row-kernel blocks per XCD: contiguous ranges of rows (neighbouring rows share B rows, which then stay
+    // in one L2), cut where the running work -- nonzeros plus a fixed cost per row -- passes each eighth.
+    {
+        const uint32_t items_per_block = 256u >> p->rows_logl;             // (row, slab) pairs of one 256-thread block
+        const uint64_t total_items = uint64_t(row_list.size()) * p->rows_slabs;
+        const uint32_t total_blocks = uint32_t((total_items + items_per_block - 1) / items_per_block);
+        uint64_t total_work = 0;
+        for (uint32_t q = 0; q < d->P; ++q)
+            if (to_rows[q]) total_work += d->panelNnz[q] + 4u * CUTE_TM;
+        uint64_t work = 0, items = 0;
+        uint32_t x = 1;
+        p->rowRanges.first[0] = 0;
+        for (uint32_t q = 0; q < d->P && x < cute_dev::kNumXcd; ++q) {
+            if (!to_rows[q]) continue;
+            work += d->panelNnz[q] + 4u * CUTE_TM;
+            items += uint64_t(CUTE_TM) * p->rows_slabs;
+            while (x < cute_dev::kNumXcd && work * cute_dev::kNumXcd >= total_work * x)
+                p->rowRanges.first[x++] = uint32_t(std::min<uint64_t>(total_blocks, (items + items_per_block - 1) / items_per_block));
+        }
+        while (x <= cute_dev::kNumXcd) p->rowRanges.first[x++] = total_blocks;
+        p->rowBlocksPerXcd = 0;
+        for (uint32_t k = 0; k < cute_dev::kNumXcd; ++k)
+            p->rowBlocksPerXcd = std::max(p->rowBlocksPerXcd, p->rowRanges.first[k + 1] - p->rowRanges.first[k]);
+    }
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
     if (rc == CUTE_OK) rc = upload(&p->dAtomicPanels, atomic_panels.data(), atomic_panels.size());
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
@@ -416,7 +446,11 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->info.path = uint32_t(t.path);
     p->info.mfmaShape = uint32_t(p->shape);
     p->info.pipeline = uint32_t(p->pipeline);
-    p->info.fusedLaunch = (p->shape == 2 && !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2) ? 1u : 0u;
+    // one launch for a mixed plan: the quad kernel with any row shape of 4-float lanes, the rolling brick
+    // kernel in the shapes the planner itself picks for N (forced column groups fall back to two launches)
+    const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
+    const bool brick_default_shape = p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
+    p->info.fusedLaunch = (rows_fusable && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
 }
@@ -448,17 +482,19 @@ void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream
 
 template <int VEC, bool BATCHED>
 void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
-                     const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
+                     const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s,
+                     const cute_dev::XcdRanges *ranges, uint32_t blocks_per_xcd)
 {
     const uint64_t lanes = (uint64_t(num_rows) * slabs) << logl;
-    // the batched kernel remaps its blocks per XCD and wants a multiple of 8 of them
+    // the batched kernel deals its blocks to the XCDs in contiguous ranges (all as long as the longest)
     const uint32_t blocks = uint32_t((lanes + 255) / 256);
-    const dim3 grid(BATCHED ? (blocks + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd * cute_dev::kNumXcd : blocks), block(256);
+    const dim3 grid(BATCHED ? blocks_per_xcd * cute_dev::kNumXcd : blocks), block(256);
+    const cute_dev::XcdRanges rg = ranges ? *ranges : cute_dev::XcdRanges{};
 #define CUTE_ROWS_CASE(LL)                                                                                        \
     case LL:                                                                                                      \
         if (BATCHED)                                                                                              \
             hipLaunchKernelGGL((cute_dev::csr_rows_batched<VEC, LL, 8>), grid, block, 0, s, row_list, num_rows,    \
-                               slabs, rp, cl, vl, dB, dC, N);                                                     \
+                               slabs, rp, cl, vl, dB, dC, N, rg);                                                 \
         else                                                                                                      \
             hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, row_list, num_rows, slabs, rp,    \
                                cl, vl, dB, dC, N);                                                                \
@@ -473,11 +509,12 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
 // batched: the library's sparse-panel kernel; otherwise the plain comparison kernel
 template <bool BATCHED>
 void launch_rows(int vec, int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
-                 const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s)
+                 const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s,
+                 const cute_dev::XcdRanges *ranges = nullptr, uint32_t blocks_per_xcd = 0)
 {
-    if (vec == 4) launch_rows_vec<4, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
-    else if (vec == 2) launch_rows_vec<2, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
-    else launch_rows_vec<1, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s);
+    if (vec == 4) launch_rows_vec<4, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s, ranges, blocks_per_xcd);
+    else if (vec == 2) launch_rows_vec<2, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s, ranges, blocks_per_xcd);
+    else launch_rows_vec<1, BATCHED>(logl, row_list, num_rows, slabs, rp, cl, vl, dB, dC, N, s, ranges, blocks_per_xcd);
 }
 
 int check_launch(const char *what)
@@ -560,6 +597,44 @@ void launch_blocked_ell(const cute_blocked_ell_dev *d, const float *dB, float *d
 }
 }  // namespace
 
+namespace {
+// Brick chunks and sparse rows in one launch.  (VEC, NG, lanes per row) follow from N the way the planner
+// picks them; returns false for a combination that is not instantiated (the caller then launches twice).
+template <int VEC, int NG, int LOG_L>
+void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s, const dim3 &grid,
+                          uint32_t per_xcd)
+{
+    const uint32_t N = p->info.N;
+    const uint64_t brick_blocks = uint64_t(grid.x) * grid.y, row_blocks = uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd;
+    const dim3 flat(uint32_t(brick_blocks + row_blocks)), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
+#define CUTE_BRICK_ROWS(F)                                                                                                \
+    hipLaunchKernelGGL((cute_dev::hrpb_brick_rows_f32<VEC, NG, F, LOG_L>), flat, block, 0, s, grid.x, uint32_t(brick_blocks),  \
+                       p->dChunks, p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), p->dRowList, \
+                       p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals,                    \
+                       dB, dC, N)
+    if (N % (16u * VEC * NG) == 0) CUTE_BRICK_ROWS(true);
+    else CUTE_BRICK_ROWS(false);
+#undef CUTE_BRICK_ROWS
+}
+
+bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+{
+    const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
+    const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+    const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs);
+    if (uint64_t(grid.x) * grid.y + uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd >= 0x7fffffffull) return false;
+    const int v = p->vec, g = p->ng, l = p->rows_logl;
+    if (v == 1 && g == 1 && l == 2) launch_brick_rows_as<1, 1, 2>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 2 && g == 1 && l == 3) launch_brick_rows_as<2, 1, 3>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 4) launch_brick_rows_as<4, 1, 4>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 5) launch_brick_rows_as<4, 1, 5>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 4 && g == 2 && l == 5) launch_brick_rows_as<4, 2, 5>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 4 && g == 2 && l == 6) launch_brick_rows_as<4, 2, 6>(p, dB, dC, s, grid, per_xcd);
+    else return false;
+    return true;
+}
+}  // namespace
+
 extern "C" {
 
 // Replaces SPMM_TC::run (spmm.cu:823-839): picks the kernel instantiation from N and
@@ -580,13 +655,12 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
         const bool full = N % 64u == 0, strips = p->d->quadRows == 4;
         // mixed plan: quad chunks and sparse rows in one launch (instantiated for 4-float lanes and 4..64 lanes per row)
-        const uint64_t row_lanes = (uint64_t(p->numRows) * p->rows_slabs) << p->rows_logl;
-        const uint64_t row_blocks = (row_lanes + 255) / 256, quad_blocks = uint64_t(grid.x) * grid.y;
+        const uint64_t row_blocks = uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd, quad_blocks = uint64_t(grid.x) * grid.y;
         if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
 #define CUTE_FUSED_LAUNCH(F, S, LL)                                                                                       \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
                        grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQCols, p->d->dQVals,  \
-                       p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
+                       p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
         case 2: CUTE_FUSED_LAUNCH(F, S, 2); break;                              \
@@ -612,14 +686,16 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         else CUTE_QUAD_LAUNCH(false, false);
 #undef CUTE_QUAD_LAUNCH
     } else if (p->info.numChunks) {
+        if (p->info.fusedLaunch && launch_brick_rows(p, dB, dC, s)) return check_launch("spmm launch");
         if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
         else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);
         else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, s);
         else launch_brick<1, 1>(p, dB, dC, s);
     }
     if (p->numRows) {
-        launch_rows<true>(p->rows_vec, p->rows_logl, p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
-                    p->d->dCsrVals, dB, dC, N, s);
+        // every row: no list needed, which takes one dependent load out of each row's chain
+        launch_rows<true>(p->rows_vec, p->rows_logl, p->numRows == p->d->M ? nullptr : p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
+                    p->d->dCsrVals, dB, dC, N, s, &p->rowRanges, p->rowBlocksPerXcd);
     }
     return check_launch("spmm launch");
 }

@@ -40,6 +40,19 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t gro
     return (bid % kNumXcd) * groups_per_xcd + bid / kNumXcd;
 }
 
+// The same idea with ranges of unequal length (balanced by work, not by count): XCD x owns the
+// logical blocks [first[x], first[x+1]); the launch has kNumXcd * (longest range) blocks.
+struct XcdRanges {
+    uint32_t first[kNumXcd + 1];
+};
+
+__device__ __forceinline__ bool xcd_range_id(const XcdRanges &r, uint32_t bid, uint32_t &logical)
+{
+    const uint32_t x = bid % kNumXcd;
+    logical = r.first[x] + bid / kNumXcd;
+    return logical < r.first[x + 1];
+}
+
 struct BlockHeader {          // one 128-byte header line as a wavefront sees it
     uint64_t bitmap[4];       // wave-uniform (scalar loads)
     uint32_t voff[4];         // wave-uniform
@@ -122,11 +135,11 @@ struct BrickItem {
 // so the slabs of one chunk run on the same XCD and share its B rows in that L2.
 template <int VEC, int NG>
 __device__ __forceinline__ BrickItem brick_item(const uint4 *__restrict__ chunks, uint32_t num_chunks,
-                                                uint32_t groups_per_xcd, uint32_t lane)
+                                                uint32_t groups_per_xcd, uint32_t lane, uint32_t block_x, uint32_t block_y)
 {
     BrickItem it;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const uint32_t chunk = xcd_contiguous_id(blockIdx.x, groups_per_xcd) * kWavesPerGroup + wave;
+    const uint32_t chunk = xcd_contiguous_id(block_x, groups_per_xcd) * kWavesPerGroup + wave;
     it.valid = chunk < num_chunks;
     if (!it.valid) return it;
     const uint4 ck = chunks[chunk];
@@ -134,7 +147,7 @@ __device__ __forceinline__ BrickItem brick_item(const uint4 *__restrict__ chunks
     it.end = __builtin_amdgcn_readfirstlane(ck.y);
     it.panel = __builtin_amdgcn_readfirstlane(ck.z);
     it.atomic = __builtin_amdgcn_readfirstlane(ck.w);
-    it.col0 = blockIdx.y * (16u * VEC * NG) + (lane & 15u) * VEC;
+    it.col0 = block_y * (16u * VEC * NG) + (lane & 15u) * VEC;
     return it;
 }
 
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     float *__restrict__ C, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, blockIdx.x, blockIdx.y);
     if (!it.valid) return;
     const uint32_t end = it.end, col0 = it.col0;
 
@@ -327,13 +340,15 @@ __device__ __forceinline__ void brick_store_lean(const BrickItem &it, const f32x
 // bricks skip their MFMAs.  NG = 2 lets one wavefront cover two column groups, which halves the
 // header traffic and shares the A-side index arithmetic between them.
 template <int VEC, int NG, bool FULL>
-__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_f32_rolling(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr,
-    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+__device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t block_y, const uint4 *__restrict__ chunks,
+                                                   uint32_t num_chunks, uint32_t groups_per_xcd,
+                                                   const uint32_t *__restrict__ hdr, const float *__restrict__ vals,
+                                                   uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
+                                                   uint32_t N)
 {
     typedef typename Vec<VEC>::type V;
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, block_x, block_y);
     if (!it.valid) return;
     const uint32_t end = it.end;
     const uint32_t row_pitch = N * 4u, col_off = it.col0 * 4u;
@@ -390,6 +405,14 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
         }
     }
     brick_store_lean<VEC, NG, FULL>(it, acc, C, N, lane);
+}
+
+template <int VEC, int NG, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_f32_rolling(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr,
+    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+{
+    brick_rolling_body<VEC, NG, FULL>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, hdr, vals, zero_index, B, C, N);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -760,32 +783,56 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
                                                         uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
                                                         const uint32_t *__restrict__ cols,
                                                         const float *__restrict__ vals, const float *__restrict__ B,
-                                                        float *__restrict__ C, uint32_t N)
+                                                        float *__restrict__ C, uint32_t N, XcdRanges ranges)
 {
-    // the grid is a multiple of the XCD count: each XCD walks one contiguous range of rows, so the B rows
-    // that neighbouring rows share stay in that XCD's L2
-    rows_batched_body<VEC, LOG_L, BATCH>(xcd_contiguous_id(blockIdx.x, gridDim.x / kNumXcd), row_list, num_rows, num_slabs,
-                                         rowPtr, cols, vals, B, C, N);
+    // each XCD walks one contiguous range of rows (ranges of equal work), so the B rows that neighbouring
+    // rows share stay in that XCD's L2
+    uint32_t block_id;
+    if (!xcd_range_id(ranges, blockIdx.x, block_id)) return;
+    rows_batched_body<VEC, LOG_L, BATCH>(block_id, row_list, num_rows, num_slabs, rowPtr, cols, vals, B, C, N);
 }
 
 // One launch for a plan that uses both the quad kernel and the row kernel: they write disjoint
 // panels, and the row kernel's short, even work fills the SIMDs that the quad kernel's long chunks
 // leave idle.  Blocks [0, quad_blocks) are the quad kernel's 2-D grid flattened (x fastest, so the
-// XCD of a block is still x % 8); the rest are the row kernel's blocks.
+// XCD of a block is still x % 8); the rest are the row kernel's blocks, dealt to the XCDs in
+// contiguous ranges like the row kernel's own launch does.
 template <bool FULL, bool STRIPS, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
     uint32_t quad_blocks_x, uint32_t quad_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols, const float *__restrict__ qvals,
-    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, const uint32_t *__restrict__ rowPtr,
-    const uint32_t *__restrict__ cols, const float *__restrict__ vals, const float *__restrict__ B, float *__restrict__ C,
-    uint32_t N)
+    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
+    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
     static_assert(kWaveSize * kWavesPerGroup == 256, "both bodies are written for 256-thread blocks");
-    if (blockIdx.x < quad_blocks)
+    if (blockIdx.x < quad_blocks) {
         quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, chunks, num_chunks, groups_per_xcd,
                                 qcols, qvals, B, C, N);
-    else
-        rows_batched_body<4, LOG_L, 8>(blockIdx.x - quad_blocks, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
+    } else {   // quad_blocks is a multiple of the XCD count, so the XCD of a row block is (its index) % 8 as well
+        uint32_t block_id;
+        if (!xcd_range_id(row_ranges, blockIdx.x - quad_blocks, block_id)) return;
+        rows_batched_body<4, LOG_L, 8>(block_id, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
+    }
+}
+
+// The same for a plan that pairs the rolling brick kernel with the row kernel.
+template <int VEC, int NG, bool FULL, int LOG_L>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_rows_f32(
+    uint32_t brick_blocks_x, uint32_t brick_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
+    uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ tile_vals, uint32_t zero_index,
+    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
+    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+{
+    if (blockIdx.x < brick_blocks) {
+        brick_rolling_body<VEC, NG, FULL>(blockIdx.x % brick_blocks_x, blockIdx.x / brick_blocks_x, chunks, num_chunks,
+                                          groups_per_xcd, hdr, tile_vals, zero_index, B, C, N);
+    } else {
+        uint32_t block_id;
+        if (!xcd_range_id(row_ranges, blockIdx.x - brick_blocks, block_id)) return;
+        rows_batched_body<4, LOG_L, 8>(block_id, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
+    }
 }
 
 // Thread per C element (inc/SPMM.cuh:898-920 restated for fp32 and a 64x4 thread tile).
