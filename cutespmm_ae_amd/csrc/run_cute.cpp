@@ -63,6 +63,18 @@ int main(int argc, char **argv)
         MTX_READER *reader = nullptr;
         HRPB *format = nullptr;
         bool from_cache = false;
+        {   // bring the HIP runtime up before anything is timed: the first device call costs tens of milliseconds
+            int cus = 0, wave = 0;
+            char arch[64];
+            cute::check(cute_device_info(&cus, &wave, arch, sizeof arch), "cute_device_info");
+            std::vector<float> host(1u << 18, 0.0f);   // the first allocation and the first copy pay for the runtime's set-up
+            void *warm = nullptr;
+            if (hipMalloc(&warm, host.size() * sizeof(float)) != hipSuccess ||
+                hipMemcpy(warm, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess ||
+                hipDeviceSynchronize() != hipSuccess)
+                throw cute::Error(CUTE_ERR_HIP, "device warm-up");
+            (void)hipFree(warm);
+        }
         auto t0 = std::chrono::steady_clock::now();
         if (!cache_file.empty()) {
             if (FILE *probe = std::fopen(cache_file.c_str(), "rb")) {
