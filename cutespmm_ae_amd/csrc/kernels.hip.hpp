@@ -368,6 +368,12 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
         {
             const LeanHeader h0 = load_lean_header(hdr, blk, lane);
             h1 = load_lean_header(hdr, min(blk + 1, end - 1), lane);
+            // h1's load must be complete before the loop is entered.  The wait in front of its first use in
+            // the loop is compiled once for both ways into the loop; were the load still in flight here (the
+            // compiler would sink it behind the operand loads below), that wait would allow only two younger
+            // loads and would drain the whole operand set on every iteration.  Waiting here costs nothing:
+            // the operand addresses below need h0, which was requested together with h1.
+            asm volatile("" ::"v"(h1.cols[0]), "v"(h1.cols[1]), "v"(h1.cols[2]), "v"(h1.cols[3]));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_off, it.col0, N);
