@@ -78,8 +78,9 @@ struct cute_hrpb_dev {
     float *dVals = nullptr;
     uint32_t *dRowPtr = nullptr, *dCols = nullptr;
     float *dCsrVals = nullptr;
-    uint32_t *dQCols = nullptr;         // quad lists: 16 columns per group
-    float *dQVals = nullptr;            // quad lists: 64 values per group
+    uint32_t *dQRecs = nullptr;         // quad lists: one record per group (16 columns, slot mask, first value)
+    float *dQVals = nullptr;            // quad lists: the occupied value slots in lane order, then 64 zeros
+    uint64_t numQuadVals = 0;
     uint64_t numGroups = 0;
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
     std::vector<uint32_t> qgp;          // host copy of the quad lists' groupPtr
@@ -130,7 +131,7 @@ void cute_hrpb_dev_free(cute_hrpb_dev *d)
     (void)hipFree(d->dRowPtr);
     (void)hipFree(d->dCols);
     (void)hipFree(d->dCsrVals);
-    (void)hipFree(d->dQCols);
+    (void)hipFree(d->dQRecs);
     (void)hipFree(d->dQVals);
     delete d;
 }
@@ -208,9 +209,29 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
             d->quadRows = ql.rowsPerList;
             d->quadPairs = ql.numPairs;
             d->qgp.assign(ql.groupPtr, ql.groupPtr + ql.numRowPanels + 1);
-            rc = upload(&d->dQCols, ql.cols, ql.numGroups * 16);
-            if (rc == CUTE_OK) rc = upload(&d->dQVals, ql.vals, ql.numGroups * 64);
-            d->bytes += ql.numGroups * (16 + 64) * 4;
+            // Device form of the lists: per group a record {16 columns, 64-bit mask of its occupied value
+            // slots, position of its first stored value, pad} and only the occupied slots' values -- slots of
+            // padding pairs and of rows a column does not touch hold zeros and are not stored.
+            std::vector<uint32_t> recs(ql.numGroups * cute_dev::kQuadRecordWords, 0u);
+            std::vector<float> packed;
+            packed.reserve(h->nnz + 64);
+            for (uint64_t g = 0; g < ql.numGroups; ++g) {
+                uint32_t *rec = recs.data() + g * cute_dev::kQuadRecordWords;
+                std::memcpy(rec, ql.cols + g * 16, 16 * sizeof(uint32_t));
+                uint64_t mask = 0;
+                rec[18] = uint32_t(packed.size());
+                for (uint32_t l = 0; l < 64; ++l) {
+                    const float v = ql.vals[g * 64 + l];
+                    if (v != 0.0f) { mask |= 1ull << l; packed.push_back(v); }
+                }
+                rec[16] = uint32_t(mask);
+                rec[17] = uint32_t(mask >> 32);
+            }
+            d->numQuadVals = packed.size();
+            packed.resize(packed.size() + 64, 0.0f);
+            rc = upload(&d->dQRecs, recs.data(), recs.size());
+            if (rc == CUTE_OK) rc = upload(&d->dQVals, packed.data(), packed.size());
+            d->bytes += recs.size() * 4 + packed.size() * 4;
             cute_quad_release(&ql);
         }
     }
@@ -320,7 +341,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             }
         p->shape = slots < 8u * bricks ? 2 : 1;
     }
-    if (p->shape == 2 && !(offsets_fit && d->numGroups * 64u * 4u <= 0xffffffffull)) p->shape = 1;
+    if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
     const uint32_t slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
     const uint32_t num_slabs = (N + slab - 1) / slab;
     if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
@@ -659,7 +680,8 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
 #define CUTE_FUSED_LAUNCH(F, S, LL)                                                                                       \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
-                       grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQCols, p->d->dQVals,  \
+                       grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,  \
+                       uint32_t(p->d->numQuadVals),                                                                  \
                        p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
@@ -679,7 +701,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         }
 #define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,        \
-                       p->d->dQCols, p->d->dQVals, dB, dC, N)
+                       p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, N)
         if (full && strips) CUTE_QUAD_LAUNCH(true, true);
         else if (full) CUTE_QUAD_LAUNCH(true, false);
         else if (strips) CUTE_QUAD_LAUNCH(false, true);

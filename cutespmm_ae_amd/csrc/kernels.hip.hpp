@@ -31,6 +31,7 @@ constexpr int kWaveSize = 64;
 constexpr int kWavesPerGroup = 4;
 constexpr int kHdrWords = 32;
 constexpr int kNumXcd = 8;
+constexpr int kQuadRecordWords = 20;   // device record of one quad-list group: 16 columns, mask lo/hi, first value, pad
 
 // Work-groups are handed to the 8 XCDs round-robin; this maps the hardware id to a
 // logical id such that each XCD walks one contiguous range of logical ids (neighbouring
@@ -454,9 +455,9 @@ __device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32
 
 template <bool FULL, bool STRIPS>
 __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint4 *__restrict__ chunks,
-                                          uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
-                                          const float *__restrict__ qvals, const float *__restrict__ B,
-                                          float *__restrict__ C, uint32_t N)
+                                          uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
+                                          const float *__restrict__ qvals, uint32_t zero_index,
+                                          const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
@@ -481,18 +482,27 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
         // Two operand sets, so every B operand is requested two groups before its MFMA: set 0 holds
         // group g, set 1 group g+1 (or a harmless re-read of the last group when there is none).
         float b0[16], b1[16], a0, a1;
-        uint32_t ca[16], cb[16];       // column lists of the groups being requested (scalar registers)
+        // records of the groups being requested (scalar registers): 16 columns, the 64-bit occupancy mask of
+        // the group's 64 value slots and the position of its first stored value
+        uint32_t ca[kQuadRecordWords], cb[kQuadRecordWords];
         const uint32_t last = g_end - 1u;
-        auto fetch_cols = [&](uint32_t (&c)[16], uint32_t grp) {
-            const uint32_t *src = qcols + size_t(min(grp, last)) * 16u;
+        auto fetch_cols = [&](uint32_t (&c)[kQuadRecordWords], uint32_t grp) {
+            const uint32_t *src = qrecs + size_t(min(grp, last)) * kQuadRecordWords;
 #pragma unroll
-            for (int p = 0; p < 16; ++p) c[p] = src[p];
+            for (int p = 0; p < kQuadRecordWords; ++p) c[p] = src[p];
         };
-        auto fetch_a = [&](uint32_t grp) { return qvals[size_t(min(grp, last)) * 64u + lane]; };
+        // only occupied slots are stored: lane L's value sits (number of occupied slots below L) behind the
+        // group's first one; an empty slot reads the zero kept behind the last value
+        auto fetch_a = [&](const uint32_t (&c)[kQuadRecordWords]) {
+            const uint64_t mask = (uint64_t(c[17]) << 32) | c[16];
+            const uint32_t rank = __builtin_amdgcn_mbcnt_hi(c[17], __builtin_amdgcn_mbcnt_lo(c[16], c[18]));
+            const uint32_t off = (__builtin_amdgcn_inverse_ballot_w64(mask) ? rank : zero_index) * 4u;
+            return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(qvals) + off);
+        };
         fetch_cols(ca, g);
         fetch_cols(cb, g + 1);
-        a0 = fetch_a(g);
-        a1 = fetch_a(g + 1);
+        a0 = fetch_a(ca);
+        a1 = fetch_a(cb);
 #pragma unroll
         for (int p = 0; p < 16; ++p) b0[p] = quad_load_b(B, ca[p], row_pitch, col_off);
 #pragma unroll
@@ -521,7 +531,7 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
             // group g from set 0; set 0 is refilled with group g+2.  The other column list is
             // asked for right after this one's first use (where it is waited for), so that wait
             // never covers a fetch just issued; it is first used 15 pairs later.
-            const float a0n = fetch_a(g + 2);
+            const float a0n = fetch_a(ca);
             __builtin_amdgcn_sched_barrier(0);
             CUTE_QUAD_ROLL(0, a0, b0, ca)
             fetch_cols(cb, g + 3);
@@ -529,7 +539,7 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
             CUTE_QUAD_ROLL_REST(a0, b0, ca)
             a0 = a0n;
             // group g+1 from set 1; set 1 is refilled with group g+3 (clamped to the last one)
-            const float a1n = fetch_a(g + 3);
+            const float a1n = fetch_a(cb);
             __builtin_amdgcn_sched_barrier(0);
             CUTE_QUAD_ROLL(0, a1, b1, cb)
             fetch_cols(ca, g + 4);
@@ -574,10 +584,10 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
 
 template <bool FULL, bool STRIPS>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols,
-    const float *__restrict__ qvals, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
+    const float *__restrict__ qvals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
-    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qcols, qvals, B, C, N);
+    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C, N);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -806,7 +816,7 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
 template <bool FULL, bool STRIPS, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
     uint32_t quad_blocks_x, uint32_t quad_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
-    uint32_t groups_per_xcd, const uint32_t *__restrict__ qcols, const float *__restrict__ qvals,
+    uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
     const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
     const float *__restrict__ B, float *__restrict__ C, uint32_t N)
@@ -814,7 +824,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f
     static_assert(kWaveSize * kWavesPerGroup == 256, "both bodies are written for 256-thread blocks");
     if (blockIdx.x < quad_blocks) {
         quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, chunks, num_chunks, groups_per_xcd,
-                                qcols, qvals, B, C, N);
+                                qrecs, qvals, zero_index, B, C, N);
     } else {   // quad_blocks is a multiple of the XCD count, so the XCD of a row block is (its index) % 8 as well
         uint32_t block_id;
         if (!xcd_range_id(row_ranges, blockIdx.x - quad_blocks, block_id)) return;
