@@ -413,6 +413,52 @@ def test_few_huge_panels_are_still_cut(cs, orc, torch_cuda):
     assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
 
 
+def _structured_csr(rng, kind, M, K):
+    """A few sparsity structures the planner treats differently (all rows sorted, distinct columns)."""
+    if kind == "uniform":
+        return random_csr(rng, M, K, density=rng.choice([0.002, 0.01, 0.05]))
+    if kind == "banded":
+        half = int(rng.choice([4, 24, 100]))
+        rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: min(2 * half, int(rng.integers(1, 12))))
+        for r in range(M):
+            s, e = int(rp[r]), int(rp[r + 1])
+            centre = int(r * K / M)
+            window = np.arange(max(0, centre - half), min(K, centre + half))
+            cl[s:e] = np.sort(rng.choice(window, e - s, replace=False))
+        return rp, cl, vl
+    if kind == "blocks":           # dense little blocks on a coarse random pattern, like a stiffness matrix
+        b = int(rng.choice([3, 6, 8]))
+        D = np.zeros((M, K), np.float32)
+        for i in range(0, M - b + 1, b):
+            for j in rng.choice(max(1, K // b), size=min(4, max(1, K // b)), replace=False):
+                D[i:i + b, j * b:(j + 1) * b] = rng.standard_normal((b, min(b, K - j * b)))
+        return csr_from_dense(D)
+    if kind == "hubs":             # a few very long rows among short ones, and some empty panels
+        long_rows = set(rng.choice(M, 3, replace=False).tolist())
+        empty = set(range(32, 64)) if M > 96 else set()
+        return random_csr(rng, M, K, row_nnz=lambda r: min(K, 700) if r in long_rows else 0 if r in empty else int(rng.integers(0, 5)))
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_planner_choices_on_varied_structures(cs, orc, torch_cuda, seed):
+    """Whatever the planner picks (kernel, tile width, fused launch, split panels), the product is right:
+    varied structures, sizes and widths through the default plan and with either MFMA shape forced."""
+    rng = np.random.default_rng(1000 + seed)
+    for kind in ("uniform", "banded", "blocks", "hubs"):
+        M = 16 * int(rng.integers(1, 70))
+        K = 16 * int(rng.integers(4, 90))
+        rp, cl, vl = _structured_csr(rng, kind, M, K)
+        h = cs.HRPB(M, K, rp, cl, vl)
+        for N in sorted(set(int(x) for x in rng.choice([1, 2, 4, 7, 8, 12, 16, 24, 32, 36, 48, 64, 72, 96, 128, 130, 160, 256, 260], 4, replace=False))):
+            B = rng.standard_normal((K, N)).astype(np.float32)
+            ref = orc.spmm_csr(rp, cl, vl, B)
+            for kw in (dict(), dict(mfma_shape=1), dict(mfma_shape=2)):
+                out, plan = _run(cs, torch_cuda, h, B, **kw)
+                err = cs.backward_error(rp, cl, vl, B, ref, out)
+                assert np.isfinite(out).all() and err <= BERR, (seed, kind, M, K, N, kw, err, plan.info)
+
+
 def test_launches_can_be_captured_in_a_graph(cs, orc, torch_cuda):
     """cute_spmm_run only enqueues kernels (zeroing included), so a caller may capture it in a HIP
     graph: every replay, with B changed in place between replays, equals the eager result."""
