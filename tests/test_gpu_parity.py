@@ -419,7 +419,7 @@ def _structured_csr(rng, kind, M, K):
         return random_csr(rng, M, K, density=rng.choice([0.002, 0.01, 0.05]))
     if kind == "banded":
         half = int(rng.choice([4, 24, 100]))
-        rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: min(2 * half, int(rng.integers(1, 12))))
+        rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: min(half, int(rng.integers(1, 12))))    # a clipped window still holds `half` columns
         for r in range(M):
             s, e = int(rp[r]), int(rp[r + 1])
             centre = int(r * K / M)
