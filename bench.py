@@ -81,6 +81,8 @@ def main():
     ap.add_argument("--path", choices=("auto", "mfma", "rows"), default="auto", help="kernel family (default: the planner's choice)")
     ap.add_argument("--mfma-shape", type=int, default=0, help="1: 16x16x4 brick kernel, 2: 4x4x1 quad kernel, 0: planner's choice")
     ap.add_argument("--pipeline", type=int, default=0, help="brick kernel variant: 1 rolling, 2 pipelined, 0: default")
+    ap.add_argument("--graph", action="store_true",
+                    help="record the K launches of the timed region into one HIP graph and replay it (launch-bound workloads)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run 10 plain device copies of 32 MiB and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -117,10 +119,24 @@ def main():
     # the timed region: exactly K steps, synchronised on both sides; HIP events on the launch
     # stream bracket the same K launches and give the average launch duration for the roofline
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    graph = None
+    if args.graph:
+        # cute_spmm_run only enqueues kernels, so the K launches can be captured once and replayed
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(args.steps):
+                plan.run(dB, dC, stream=torch.cuda.current_stream())
+        graph.replay()                                  # one untimed replay: the first one uploads the graph
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     ev0.record(stream)
-    for _ in range(args.steps):
-        plan.run(dB, dC)
+    if graph is not None:
+        graph.replay()
+    else:
+        for _ in range(args.steps):
+            plan.run(dB, dC)
     ev1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -148,6 +164,7 @@ def main():
     out = dict(metric="SpMM GFLOP/s (2*nnz*N/t) on 1 MI355X", value=value, unit="GFLOP/s", n_gpus=1,
                steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
                scaling="weak", vs_baseline=None, dtype="f32", data="synthetic (seeded generator)",
+               launch="hip graph replay" if args.graph else "stream launches",
                config=dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, blocks=h.numBlocks,
                            bricks=h.num_bricks, plan={k: plan.info[k] for k in
                                                       ("slabWidth", "numSlabs", "numChunks", "numAtomicChunks",
