@@ -148,12 +148,12 @@ def main():
     abytes = algorithmic_bytes(A.M, A.K, N, A.nnz)
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     kernels = []
-    if plan.info["numAtomicChunks"]:
-        kernels.append("zero_panels")
     if plan.info["numChunks"]:
         kernels.append(plan.kernel_name)
     if (plan.info["numRowPanelsSparse"] or plan.info["numEmptyPanels"]) and not plan.info["fusedLaunch"]:
         kernels.append("csr_rows_batched")
+    if plan.info["numAtomicChunks"]:
+        kernels.append("reduce_partials")
     roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                     traffic=recorded_traffic(cfg["name"]), kernel=plan.kernel_name if plan.info["numChunks"] else "csr_rows_batched",
                     kernels_per_step=kernels, kernel_ms=kernel_ms, kernel_ms_single_bracketed_median=float(np.median(each)),

@@ -14,8 +14,7 @@ HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc
 
 # -packed-fp32-ops is switched off for device code: the compiler then never forms
 # v_pk_{add,mul,fma}_f32 from scalar float code.
-DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                "-munsafe-fp-atomics"]
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
           "-pthread"]
 

@@ -100,9 +100,11 @@ struct cute_spmm_plan {
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
-    uint32_t *dAtomicPanels = nullptr;
-    uint32_t numAtomicPanels = 0;
-    uint32_t atomicPanelRows = CUTE_TM; // rows of one entry of dAtomicPanels
+    // panels (or 4-row strips) cut into several chunks: each chunk stores a partial tile, reduce_partials adds them
+    uint4 *dFixups = nullptr;           // {panel or strip, first piece, pieces, -}
+    uint32_t numFixups = 0;
+    uint32_t unitRows = CUTE_TM;        // rows of one panel / strip / piece
+    float *dPartials = nullptr;         // pieces x unitRows rows of N floats; owned by the plan, so a plan runs on one stream at a time
     uint32_t *dRowList = nullptr;
     uint32_t numRows = 0;
     cute_dev::XcdRanges rowRanges{};   // row-kernel blocks of each XCD, balanced by nonzeros
@@ -253,7 +255,8 @@ void cute_spmm_plan_free(cute_spmm_plan *p)
 {
     if (!p) return;
     (void)hipFree(p->dChunks);
-    (void)hipFree(p->dAtomicPanels);
+    (void)hipFree(p->dFixups);
+    (void)hipFree(p->dPartials);
     (void)hipFree(p->dRowList);
     delete p;
 }
@@ -396,28 +399,32 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             for (uint32_t cs = s; cs < e; cs += step) quads.insert(quads.end(), {cs, std::min(e, cs + step), q, 1u});
         }
     }
+    // A chunk of a cut panel carries the 1-based number of its partial tile; the pieces of one panel are
+    // consecutive (panels ascend through the list), and one fixup entry per cut panel adds them up afterwards.
     std::vector<uint4> chunks;
-    std::vector<uint32_t> atomic_panels;
-    uint32_t n_atomic = 0;
+    std::vector<uint4> fixups;
+    uint32_t n_pieces = 0;
     for (size_t i = 0; i + 3 < quads.size(); i += 4) {
         const uint32_t s = quads[i], e = quads[i + 1], pan = quads[i + 2];
-        uint32_t atomic = quads[i + 3];
+        uint32_t cut = quads[i + 3];
         if (to_rows[pan / upp]) continue;
         const uint32_t len = e - s;
         const uint32_t cap = t.max_chunk_blocks ? t.max_chunk_blocks : len;
-        if (len > cap) atomic = 1;                 // cut further than the partition asked for
+        if (len > cap) cut = 1;                    // cut further than the partition asked for
         const uint32_t step = std::min(cap, len);
-        if (atomic && (atomic_panels.empty() || atomic_panels.back() != pan)) atomic_panels.push_back(pan);
         for (uint32_t cs = s; cs < e; cs += step) {
-            chunks.push_back(make_uint4(cs, std::min(e, cs + step), pan, atomic));
-            n_atomic += atomic;
+            if (cut) {
+                if (fixups.empty() || fixups.back().x != pan) fixups.push_back(make_uint4(pan, n_pieces, 0u, 0u));
+                fixups.back().z++;
+                ++n_pieces;
+            }
+            chunks.push_back(make_uint4(cs, std::min(e, cs + step), pan, cut ? n_pieces : 0u));
         }
     }
     // a strip without pairs inside an MFMA-routed panel still has to be written (as zeros): an empty chunk
     if (upp > 1)
         for (uint32_t q = 0; q < num_units; ++q)
             if (unit[q] == unit[q + 1] && !to_rows[q / upp]) chunks.push_back(make_uint4(unit[q], unit[q], q, 0u));
-    // panels ascend through the chunk list, so each atomic panel is listed (and zeroed) once
     std::vector<uint32_t> row_list;
     for (uint32_t q = 0; q < d->P; ++q)
         if (to_rows[q])
@@ -448,17 +455,23 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             p->rowBlocksPerXcd = std::max(p->rowBlocksPerXcd, p->rowRanges.first[k + 1] - p->rowRanges.first[k]);
     }
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
-    if (rc == CUTE_OK) rc = upload(&p->dAtomicPanels, atomic_panels.data(), atomic_panels.size());
+    if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
+    p->unitRows = CUTE_TM / upp;
+    if (rc == CUTE_OK && n_pieces) {
+        // the kernels address the partial tiles like C, with 32-bit byte offsets
+        const uint64_t bytes = uint64_t(n_pieces) * p->unitRows * N * sizeof(float);
+        if (bytes > 0xffffffffull) rc = CUTE_ERR_NOMEM;
+        else if (hipMalloc(reinterpret_cast<void **>(&p->dPartials), bytes) != hipSuccess) rc = CUTE_ERR_NOMEM;
+    }
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
-    p->numAtomicPanels = uint32_t(atomic_panels.size());
-    p->atomicPanelRows = CUTE_TM / upp;
+    p->numFixups = uint32_t(fixups.size());
     p->numRows = uint32_t(row_list.size());
     p->info.N = N;
     p->info.slabWidth = slab;
     p->info.numSlabs = num_slabs;
     p->info.numChunks = uint32_t(chunks.size());
-    p->info.numAtomicChunks = n_atomic;
+    p->info.numAtomicChunks = n_pieces;      // chunks of cut panels (the field keeps its name from the atomics they once used)
     p->info.numBrickPanels = n_brick;
     p->info.numRowPanelsSparse = n_rows;
     p->info.numEmptyPanels = n_empty;
@@ -488,10 +501,10 @@ void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipS
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
     if (p->pipeline == 1)
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, NG, FULL>), grid, block, 0, s, p->dChunks,
-                           p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, p->info.N);
+                           p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, p->dPartials, p->info.N);
     else
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), grid, block, 0, s, p->dChunks, p->info.numChunks,
-                           per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->info.N);
+                           per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->dPartials, p->info.N);
 }
 
 template <int VEC, int NG>
@@ -632,7 +645,7 @@ void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, h
     hipLaunchKernelGGL((cute_dev::hrpb_brick_rows_f32<VEC, NG, F, LOG_L>), flat, block, 0, s, grid.x, uint32_t(brick_blocks),  \
                        p->dChunks, p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), p->dRowList, \
                        p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals,                    \
-                       dB, dC, N)
+                       dB, dC, p->dPartials, N)
     if (N % (16u * VEC * NG) == 0) CUTE_BRICK_ROWS(true);
     else CUTE_BRICK_ROWS(false);
 #undef CUTE_BRICK_ROWS
@@ -666,10 +679,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
     if ((reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC)) & 15u) return CUTE_ERR_ARG;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t N = p->info.N;
-    if (p->numAtomicPanels) {
-        hipLaunchKernelGGL(cute_dev::zero_panels, dim3(p->numAtomicPanels), dim3(256), 0, s, p->dAtomicPanels,
-                           p->numAtomicPanels, p->atomicPanelRows, dC, N);
-    }
+    bool rows_launched = false;        // the sparse rows went out together with the MFMA chunks
     if (p->info.numChunks && p->shape == 2) {
         const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
         const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
@@ -682,7 +692,8 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
     hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
                        grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,  \
                        uint32_t(p->d->numQuadVals),                                                                  \
-                       p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC, N)
+                       p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC,    \
+                       p->dPartials, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
         case 2: CUTE_FUSED_LAUNCH(F, S, 2); break;                              \
@@ -697,28 +708,35 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
             else { CUTE_FUSED_LL(false, false) }
 #undef CUTE_FUSED_LL
 #undef CUTE_FUSED_LAUNCH
-            return check_launch("spmm launch");
-        }
+            rows_launched = true;
+        } else {
 #define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,        \
-                       p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, N)
+                       p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, p->dPartials, N)
         if (full && strips) CUTE_QUAD_LAUNCH(true, true);
         else if (full) CUTE_QUAD_LAUNCH(true, false);
         else if (strips) CUTE_QUAD_LAUNCH(false, true);
         else CUTE_QUAD_LAUNCH(false, false);
 #undef CUTE_QUAD_LAUNCH
+        }
     } else if (p->info.numChunks) {
-        if (p->info.fusedLaunch && launch_brick_rows(p, dB, dC, s)) return check_launch("spmm launch");
-        if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
+        if (p->info.fusedLaunch && launch_brick_rows(p, dB, dC, s)) rows_launched = true;
+        else if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
         else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);
         else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, s);
         else launch_brick<1, 1>(p, dB, dC, s);
     }
-    if (p->numRows) {
+    if (p->numRows && !rows_launched) {
         // every row: no list needed, which takes one dependent load out of each row's chain
         launch_rows<true>(p->rows_vec, p->rows_logl, p->numRows == p->d->M ? nullptr : p->dRowList, p->numRows, p->rows_slabs, p->d->dRowPtr, p->d->dCols,
                     p->d->dCsrVals, dB, dC, N, s, &p->rowRanges, p->rowBlocksPerXcd);
     }
+    // panels that were cut: add their partial tiles up, in chunk order (no atomics, so a product is
+    // the same bit for bit every time it is computed)
+    if (p->numFixups)
+        hipLaunchKernelGGL(cute_dev::reduce_partials, dim3(p->numFixups, (p->unitRows * N + 63u) / 64u),
+                           dim3(cute_dev::kWaveSize * cute_dev::kReduceWaves), 0, s, p->dFixups, p->numFixups, p->unitRows,
+                           p->dPartials, dC, N);
     return check_launch("spmm launch");
 }
 

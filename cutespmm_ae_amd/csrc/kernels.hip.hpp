@@ -120,14 +120,16 @@ __device__ __forceinline__ void mfma_block(const BlockOperands<VEC, NG> &o, f32x
     }
 }
 
-// chunks[i] = {first block, end block, row panel, atomic}.  A work item is (chunk, slab);
+// chunks[i] = {first block, end block, row panel, piece}.  piece = 0: the chunk is its panel's only one and
+// stores the C tile; piece = k > 0: the panel is cut, and this chunk stores its partial tile as "panel" k-1
+// of the partials matrix (same row pitch as C), which reduce_partials adds up afterwards.  A work item is (chunk, slab);
 // slab s covers columns [s*16*VEC*NG, (s+1)*16*VEC*NG).  Lane L = 16*g + j owns, inside
 // column group ng, the VEC consecutive columns starting at s*slab + ng*16*VEC + j*VEC;
 // MFMA tile v of that group therefore holds the columns {.. + j*VEC + v}, and after the
 // MFMA lane L holds rows 4g..4g+3 of exactly those VEC columns -> one vector store per row.
 // FULL: N is a multiple of the slab width, so no column guard is compiled in.
 struct BrickItem {
-    uint32_t start, end, panel, atomic, col0;
+    uint32_t start, end, panel, piece, col0;
     bool valid;
 };
 
@@ -147,33 +149,29 @@ __device__ __forceinline__ BrickItem brick_item(const uint4 *__restrict__ chunks
     it.start = __builtin_amdgcn_readfirstlane(ck.x);
     it.end = __builtin_amdgcn_readfirstlane(ck.y);
     it.panel = __builtin_amdgcn_readfirstlane(ck.z);
-    it.atomic = __builtin_amdgcn_readfirstlane(ck.w);
+    it.piece = __builtin_amdgcn_readfirstlane(ck.w);
     it.col0 = block_y * (16u * VEC * NG) + (lane & 15u) * VEC;
     return it;
 }
 
 template <int VEC, int NG, bool FULL>
 __device__ __forceinline__ void brick_store(const BrickItem &it, const f32x4 (&acc)[NG][VEC], float *__restrict__ C,
-                                            uint32_t N, uint32_t lane)
+                                            float *__restrict__ partials, uint32_t N, uint32_t lane)
 {
     typedef typename Vec<VEC>::type V;
-    const uint32_t row0 = it.panel * 16u + (lane >> 4) * 4u;
+    float *out_base = it.piece ? partials : C;
+    const uint32_t row0 = (it.piece ? it.piece - 1u : it.panel) * 16u + (lane >> 4) * 4u;
 #pragma unroll
     for (int ng = 0; ng < NG; ++ng) {
         const uint32_t c = it.col0 + uint32_t(ng) * 16u * VEC;
         if (!FULL && c >= N) continue;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float *dst = C + size_t(row0 + r) * N + c;
-            if (it.atomic) {
+            float *dst = out_base + size_t(row0 + r) * N + c;
+            V out;
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
-            } else {
-                V out;
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
-                __builtin_nontemporal_store(out, reinterpret_cast<V *>(dst));   // C is not read again: keep it out of the L2
-            }
+            for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
+            __builtin_nontemporal_store(out, reinterpret_cast<V *>(dst));   // not read again by this launch: keep it out of the L2
         }
     }
 }
@@ -185,7 +183,7 @@ template <int VEC, int NG, bool FULL>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd,
     const uint32_t *__restrict__ hdr, const float *__restrict__ vals, const float *__restrict__ B,
-    float *__restrict__ C, uint32_t N)
+    float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, blockIdx.x, blockIdx.y);
@@ -250,7 +248,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup) void hrpb_brick_f32(
         __builtin_amdgcn_sched_barrier(0);
         mfma_block<VEC, NG>(opA, acc, lane);
     }
-    brick_store<VEC, NG, FULL>(it, acc, C, N, lane);
+    brick_store<VEC, NG, FULL>(it, acc, C, partials, N, lane);
 }
 
 // One brick's loads -- the unit of the rolling pipeline below -- written for a SIMD whose
@@ -309,10 +307,11 @@ __device__ __forceinline__ void load_brick_lean(typename Vec<VEC>::type (&b_out)
 // C tile of one item, addressed like the loads: 32-bit byte offsets from a scalar base.
 template <int VEC, int NG, bool FULL>
 __device__ __forceinline__ void brick_store_lean(const BrickItem &it, const f32x4 (&acc)[NG][VEC], float *__restrict__ C,
-                                                 uint32_t N, uint32_t lane)
+                                                 float *__restrict__ partials, uint32_t N, uint32_t lane)
 {
     typedef typename Vec<VEC>::type V;
-    const uint32_t row0 = it.panel * 16u + (lane >> 4) * 4u;
+    char *out_base = reinterpret_cast<char *>(it.piece ? partials : C);
+    const uint32_t row0 = (it.piece ? it.piece - 1u : it.panel) * 16u + (lane >> 4) * 4u;
 #pragma unroll
     for (int ng = 0; ng < NG; ++ng) {
         const uint32_t c = it.col0 + uint32_t(ng) * 16u * VEC;
@@ -320,16 +319,10 @@ __device__ __forceinline__ void brick_store_lean(const BrickItem &it, const f32x
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const uint32_t off = __umul24(row0 + r, N * 4u) + c * 4u;
-            float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-            if (it.atomic) {
+            V out;
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) unsafeAtomicAdd(dst + v, acc[ng][v][r]);
-            } else {
-                V out;
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
-                __builtin_nontemporal_store(out, reinterpret_cast<V *>(dst));   // C is not read again: keep it out of the L2
-            }
+            for (int v = 0; v < VEC; ++v) vec_set<VEC>(out, v, acc[ng][v][r]);
+            __builtin_nontemporal_store(out, reinterpret_cast<V *>(out_base + off));   // not read again by this launch
         }
     }
 }
@@ -345,7 +338,7 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
                                                    uint32_t num_chunks, uint32_t groups_per_xcd,
                                                    const uint32_t *__restrict__ hdr, const float *__restrict__ vals,
                                                    uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
-                                                   uint32_t N)
+                                                   float *__restrict__ partials, uint32_t N)
 {
     typedef typename Vec<VEC>::type V;
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
@@ -411,15 +404,17 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
                     acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], vec_get<VEC>(b[j][ng], v), acc[ng][v], 0, 0, 0);
         }
     }
-    brick_store_lean<VEC, NG, FULL>(it, acc, C, N, lane);
+    brick_store_lean<VEC, NG, FULL>(it, acc, C, partials, N, lane);
 }
 
 template <int VEC, int NG, bool FULL>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_f32_rolling(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr,
-    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
+    float *__restrict__ partials, uint32_t N)
 {
-    brick_rolling_body<VEC, NG, FULL>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, hdr, vals, zero_index, B, C, N);
+    brick_rolling_body<VEC, NG, FULL>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, hdr, vals, zero_index, B, C,
+                                      partials, N);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -437,7 +432,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
 // each, a contiguous 256-byte piece of a B row.  Two operand sets roll: as soon as the MFMA of
 // pair p is issued, B operand p of the group after next is requested into the same register.
 //
-// chunks[i] = {first group, end group, row panel (or 4-row strip), atomic}; launch: x walks
+// chunks[i] = {first group, end group, row panel (or 4-row strip), piece} (piece as for the brick kernels); launch: x walks
 // the chunks, y the slabs.  STRIPS: one list per 4-row strip (cute_quad_build_strips) instead of four
 // lockstep lists per panel; the instruction stream is the same, only the accumulators mean something else.
 // Addresses are 32-bit byte offsets from scalar bases; the planner checks the sizes.
@@ -457,7 +452,8 @@ template <bool FULL, bool STRIPS>
 __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint4 *__restrict__ chunks,
                                           uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
                                           const float *__restrict__ qvals, uint32_t zero_index,
-                                          const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+                                          const float *__restrict__ B, float *__restrict__ C,
+                                          float *__restrict__ partials, uint32_t N)
 {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
@@ -466,7 +462,7 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
     const uint4 ck = chunks[chunk];
     const uint32_t g_end = __builtin_amdgcn_readfirstlane(ck.y);
     const uint32_t panel = __builtin_amdgcn_readfirstlane(ck.z);
-    const uint32_t atomic = __builtin_amdgcn_readfirstlane(ck.w);
+    const uint32_t piece = __builtin_amdgcn_readfirstlane(ck.w);
     uint32_t g = __builtin_amdgcn_readfirstlane(ck.x);
 
     const uint32_t n = block_y * kWaveSize + lane;
@@ -555,27 +551,27 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
 #undef CUTE_QUAD_MFMA16
     }
     if (live) {
+        // a cut panel's chunk stores its tile into the partials matrix instead (rows (piece-1)*16.., same pitch)
+        char *out_base = reinterpret_cast<char *>(piece ? partials : C);
+        const uint32_t out_unit = piece ? piece - 1u : panel;
         if (STRIPS) {
             // all 16 pairs of a group belong to one 4-row strip; the four accumulators only break
             // the dependency chain and are summed here
             const f32x4 sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-            uint32_t off = __umul24(panel * 4u, row_pitch) + n * 4u;
+            uint32_t off = __umul24(out_unit * 4u, row_pitch) + n * 4u;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                if (atomic) unsafeAtomicAdd(dst, sum[i]);
-                else __builtin_nontemporal_store(sum[i], dst);
+                __builtin_nontemporal_store(sum[i], reinterpret_cast<float *>(out_base + off));
                 off += row_pitch;
             }
         } else {
-            uint32_t off = __umul24(panel * 16u, row_pitch) + n * 4u;
+            uint32_t off = __umul24(out_unit * 16u, row_pitch) + n * 4u;
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float *dst = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                    if (atomic) unsafeAtomicAdd(dst, acc[rg][i]);
-                    else __builtin_nontemporal_store(acc[rg][i], dst);   // C is not read again: keep it out of the L2
+                    // not read again by this launch: keep it out of the L2
+                    __builtin_nontemporal_store(acc[rg][i], reinterpret_cast<float *>(out_base + off));
                     off += row_pitch;
                 }
         }
@@ -585,9 +581,11 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
 template <bool FULL, bool STRIPS>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
     const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
-    const float *__restrict__ qvals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+    const float *__restrict__ qvals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
+    float *__restrict__ partials, uint32_t N)
 {
-    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C, N);
+    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C,
+                            partials, N);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -695,14 +693,42 @@ __global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict
     }
 }
 
-// Zero the C rows of the listed panels (16 rows) or strips (4 rows): those whose chunks combine through atomics.
-__global__ void zero_panels(const uint32_t *__restrict__ panels, uint32_t count, uint32_t rows_per_panel,
-                            float *__restrict__ C, uint32_t N)
+// Adds up the partial tiles of the panels (16 rows) or strips (4 rows) that were cut into several chunks:
+// fixups[i] = {panel or strip, first piece, number of pieces, -}; piece k is rows [k*rows, (k+1)*rows) of the
+// partials matrix, whose row pitch is N like C's.  Block (i, j) handles 64 consecutive elements of tile i:
+// wavefront w adds the pieces w, w+16, w+32, ... (independent loads, a few at a time), then the sixteen sums
+// are added in wavefront order.  The order is fixed, so the result does not depend on which chunk finished
+// first -- the same product gives the same bits every time.
+constexpr int kReduceWaves = 16;
+
+__global__ __launch_bounds__(kWaveSize *kReduceWaves) void reduce_partials(const uint4 *__restrict__ fixups, uint32_t count,
+                                                                           uint32_t rows, const float *__restrict__ partials,
+                                                                           float *__restrict__ C, uint32_t N)
 {
-    const uint32_t p = blockIdx.x;
-    if (p >= count) return;
-    float *base = C + size_t(panels[p]) * rows_per_panel * N;
-    for (uint32_t i = threadIdx.x; i < rows_per_panel * N; i += blockDim.x) base[i] = 0.0f;
+    __shared__ float sums[kReduceWaves][kWaveSize];
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
+    if (blockIdx.x >= count) return;
+    const uint4 fx = fixups[blockIdx.x];
+    const uint32_t tile = rows * N;
+    const uint32_t e = blockIdx.y * kWaveSize + lane;
+    const bool valid = e < tile;
+    const float *src = partials + size_t(fx.y) * tile + (valid ? e : 0u);
+    float sum = 0.0f;
+    uint32_t k = wave;
+    for (; k + 3u * kReduceWaves < fx.z; k += 4u * kReduceWaves) {
+        const float p0 = src[size_t(k) * tile], p1 = src[size_t(k + kReduceWaves) * tile];
+        const float p2 = src[size_t(k + 2u * kReduceWaves) * tile], p3 = src[size_t(k + 3u * kReduceWaves) * tile];
+        sum = (((sum + p0) + p1) + p2) + p3;
+    }
+    for (; k < fx.z; k += kReduceWaves) sum += src[size_t(k) * tile];
+    sums[wave][lane] = sum;
+    __syncthreads();
+    if (wave == 0 && valid) {
+        float total = sums[0][lane];
+#pragma unroll
+        for (int w = 1; w < kReduceWaves; ++w) total += sums[w][lane];
+        __builtin_nontemporal_store(total, C + size_t(fx.x) * tile + e);
+    }
 }
 
 // One group of L = 1<<LOG_L lanes per row; lane t of the group owns VEC consecutive columns
@@ -819,12 +845,12 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f
     uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
     const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
-    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+    const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
     static_assert(kWaveSize * kWavesPerGroup == 256, "both bodies are written for 256-thread blocks");
     if (blockIdx.x < quad_blocks) {
         quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, chunks, num_chunks, groups_per_xcd,
-                                qrecs, qvals, zero_index, B, C, N);
+                                qrecs, qvals, zero_index, B, C, partials, N);
     } else {   // quad_blocks is a multiple of the XCD count, so the XCD of a row block is (its index) % 8 as well
         uint32_t block_id;
         if (!xcd_range_id(row_ranges, blockIdx.x - quad_blocks, block_id)) return;
@@ -839,11 +865,11 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
     uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ tile_vals, uint32_t zero_index,
     const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
-    const float *__restrict__ B, float *__restrict__ C, uint32_t N)
+    const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
     if (blockIdx.x < brick_blocks) {
         brick_rolling_body<VEC, NG, FULL>(blockIdx.x % brick_blocks_x, blockIdx.x / brick_blocks_x, chunks, num_chunks,
-                                          groups_per_xcd, hdr, tile_vals, zero_index, B, C, N);
+                                          groups_per_xcd, hdr, tile_vals, zero_index, B, C, partials, N);
     } else {
         uint32_t block_id;
         if (!xcd_range_id(row_ranges, blockIdx.x - brick_blocks, block_id)) return;

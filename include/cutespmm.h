@@ -325,13 +325,13 @@ typedef struct cute_plan_info {
     uint32_t slabWidth;        /* columns of C per work item                              */
     uint32_t numSlabs;
     uint32_t numChunks;        /* brick-kernel work items along the panel axis            */
-    uint32_t numAtomicChunks;  /* of which combine through atomics                        */
+    uint32_t numAtomicChunks;  /* of which are pieces of cut panels (partial tiles, added up by a second kernel; the name dates from atomics) */
     uint32_t numBrickPanels, numRowPanelsSparse, numEmptyPanels;
     uint32_t slots;
     uint32_t precision, path;
     uint32_t mfmaShape;        /* MFMA kernel in use: 1 16x16x4 bricks, 2 4x4x1 quad lists */
     uint32_t pipeline;         /* brick kernel variant in use: 1 rolling, 2 pipelined     */
-    uint32_t fusedLaunch;      /* 1: quad chunks and sparse rows go out as one launch     */
+    uint32_t fusedLaunch;      /* 1: MFMA chunks and sparse rows go out as one launch     */
     uint32_t reserved[2];
 } cute_plan_info;
 
@@ -342,7 +342,10 @@ int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out);
 void cute_spmm_plan_free(cute_spmm_plan *p);
 /* dB [K x N], dC [M x N]: device pointers, row-major, 16-byte aligned.  Asynchronous on
  * `stream` (a hipStream_t, NULL = default stream).  C is fully overwritten: the caller
- * need not zero it (the reference requires cudaMemset first, run.cu:43,49). */
+ * need not zero it (the reference requires cudaMemset first, run.cu:43,49).  No atomics are
+ * used, so equal inputs give equal bits.  A plan whose panels were cut (numAtomicChunks > 0)
+ * keeps their partial tiles in a buffer of its own: launches of ONE plan must not overlap in
+ * time (same stream, or ordered by events); different plans are independent. */
 int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
 
 /* ------------------------------------------------------------------------------------

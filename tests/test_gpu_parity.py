@@ -151,7 +151,7 @@ def test_edge_shapes(cs, orc, torch_cuda):
             assert (out[np.diff(rp.astype(np.int64)) == 0] == 0).all()      # empty rows are written as zeros
 
 
-def test_split_panels_combine_through_atomics(cs, orc, torch_cuda):
+def test_split_panels_add_up(cs, orc, torch_cuda):
     """A few very long panels among short ones: the planner cuts them and the pieces add up."""
     rng = np.random.default_rng(8)
     M, K, N = 512, 4096, 128
@@ -167,15 +167,23 @@ def test_split_panels_combine_through_atomics(cs, orc, torch_cuda):
         for kw in (dict(max_chunk_blocks=1), dict(max_chunk_blocks=3), dict(slots=64), dict(slots=864)):
             out, plan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=shape, **kw)
             assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (shape, kw)
-    # a second launch on the same output buffer must not accumulate on top of the first
+    # a second launch on the same output buffer must not accumulate on top of the first, and the pieces of a
+    # cut panel are added in a fixed order: the same product gives the same bits every time
     import torch
     dB = torch.from_numpy(B).cuda()
-    dC = torch.zeros((M, N), device="cuda")
-    plan = cs.SPMM_TC(h, N, path=cs.PATH_BRICK, max_chunk_blocks=2)
-    plan.run(dB, dC)
-    plan.run(dB, dC)
-    torch.cuda.synchronize()
-    assert cs.backward_error(rp, cl, vl, B, ref, dC.cpu().numpy()) <= BERR
+    for shape in (1, 2):
+        dC = torch.zeros((M, N), device="cuda")
+        plan = cs.SPMM_TC(h, N, path=cs.PATH_BRICK, mfma_shape=shape, max_chunk_blocks=2)
+        plan.run(dB, dC)
+        plan.run(dB, dC)
+        torch.cuda.synchronize()
+        first = dC.cpu().numpy().copy()
+        assert cs.backward_error(rp, cl, vl, B, ref, first) <= BERR
+        for _ in range(3):
+            dC.fill_(float("nan"))
+            plan.run(dB, dC)
+            torch.cuda.synchronize()
+            assert (dC.cpu().numpy() == first).all()
 
 
 def test_csr_comparison_kernels(cs, orc, torch_cuda):
@@ -344,7 +352,7 @@ def test_full_size_other_configs(cs, orc, torch_cuda, cfg):
 
 def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
     """The quad kernel on one list per 4-row strip (forced, and chosen by the library for a matrix
-    with a few very long rows), including split strips that combine through atomics."""
+    with a few very long rows), including strips that are cut into several chunks."""
     torch = torch_cuda
     rng = np.random.default_rng(21)
     M, K = 512, 4096
@@ -465,7 +473,7 @@ def test_launches_can_be_captured_in_a_graph(cs, orc, torch_cuda):
     torch = torch_cuda
     rng = np.random.default_rng(9)
     M, K, N = 512, 4096, 128
-    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1200 if r in (5, 300) else 6)     # split panels: atomics + zeroing
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1200 if r in (5, 300) else 6)     # cut panels: partial tiles + the reduce kernel
     h = cs.HRPB(M, K, rp, cl, vl)
     for kw in (dict(), dict(path=cs.PATH_BRICK, mfma_shape=1), dict(path=cs.PATH_BRICK, mfma_shape=2)):
         plan = cs.SPMM_TC(h, N, **kw)
