@@ -695,10 +695,12 @@ __global__ __launch_bounds__(256) void blocked_ell_f32(const int32_t *__restrict
 
 // Adds up the partial tiles of the panels (16 rows) or strips (4 rows) that were cut into several chunks:
 // fixups[i] = {panel or strip, first piece, number of pieces, -}; piece k is rows [k*rows, (k+1)*rows) of the
-// partials matrix, whose row pitch is N like C's.  Block (i, j) handles 64 consecutive elements of tile i:
-// wavefront w adds the pieces w, w+16, w+32, ... (independent loads, a few at a time), then the sixteen sums
-// are added in wavefront order.  The order is fixed, so the result does not depend on which chunk finished
-// first -- the same product gives the same bits every time.
+// partials matrix, whose row pitch is N like C's.  A block of sixteen wavefronts works on tile i in segments
+// of 64 elements.  With few pieces every wavefront takes a segment of its own; with many, G = 2..16
+// wavefronts share a segment, wavefront g adding the pieces g, g+G, g+2G, ... (independent loads, four at a
+// time), and their sums are then added in wavefront order.  G depends on the piece count alone and every
+// order is fixed, so the result does not depend on which chunk finished first: the same product gives the
+// same bits every time.  The launch has one block per (tile, segment); blocks past the last segment group exit.
 constexpr int kReduceWaves = 16;
 
 __global__ __launch_bounds__(kWaveSize *kReduceWaves) void reduce_partials(const uint4 *__restrict__ fixups, uint32_t count,
@@ -706,29 +708,35 @@ __global__ __launch_bounds__(kWaveSize *kReduceWaves) void reduce_partials(const
                                                                            float *__restrict__ C, uint32_t N)
 {
     __shared__ float sums[kReduceWaves][kWaveSize];
-    const uint32_t lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
     if (blockIdx.x >= count) return;
     const uint4 fx = fixups[blockIdx.x];
+    const uint32_t pieces = __builtin_amdgcn_readfirstlane(fx.z);
+    const uint32_t G = pieces <= 4 ? 1u : pieces <= 8 ? 2u : pieces <= 16 ? 4u : pieces <= 32 ? 8u : 16u;
+    const uint32_t segs_per_block = kReduceWaves / G;
     const uint32_t tile = rows * N;
-    const uint32_t e = blockIdx.y * kWaveSize + lane;
+    if (blockIdx.y * segs_per_block * kWaveSize >= tile) return;      // whole block: nothing left of this tile
+    const uint32_t seg = blockIdx.y * segs_per_block + wave / G, g = wave % G;
+    const uint32_t e = seg * kWaveSize + lane;
     const bool valid = e < tile;
     const float *src = partials + size_t(fx.y) * tile + (valid ? e : 0u);
     float sum = 0.0f;
-    uint32_t k = wave;
-    for (; k + 3u * kReduceWaves < fx.z; k += 4u * kReduceWaves) {
-        const float p0 = src[size_t(k) * tile], p1 = src[size_t(k + kReduceWaves) * tile];
-        const float p2 = src[size_t(k + 2u * kReduceWaves) * tile], p3 = src[size_t(k + 3u * kReduceWaves) * tile];
+    uint32_t k = g;
+    for (; k < pieces; k += 4u * G) {          // four loads in flight; a piece past the end counts as zero
+        const float p0 = src[size_t(k) * tile];
+        const float p1 = k + G < pieces ? src[size_t(k + G) * tile] : 0.0f;
+        const float p2 = k + 2u * G < pieces ? src[size_t(k + 2u * G) * tile] : 0.0f;
+        const float p3 = k + 3u * G < pieces ? src[size_t(k + 3u * G) * tile] : 0.0f;
         sum = (((sum + p0) + p1) + p2) + p3;
     }
-    for (; k < fx.z; k += kReduceWaves) sum += src[size_t(k) * tile];
-    sums[wave][lane] = sum;
-    __syncthreads();
-    if (wave == 0 && valid) {
-        float total = sums[0][lane];
-#pragma unroll
-        for (int w = 1; w < kReduceWaves; ++w) total += sums[w][lane];
-        __builtin_nontemporal_store(total, C + size_t(fx.x) * tile + e);
+    if (G > 1) {
+        sums[wave][lane] = sum;
+        __syncthreads();
+        if (g != 0) return;
+        for (uint32_t w = 1; w < G; ++w) sum += sums[wave + w][lane];
     }
+    if (valid) __builtin_nontemporal_store(sum, C + size_t(fx.x) * tile + e);
 }
 
 // One group of L = 1<<LOG_L lanes per row; lane t of the group owns VEC consecutive columns
