@@ -310,12 +310,12 @@ typedef enum cute_precision {
 typedef struct cute_tunables {
     int32_t path;              /* cute_path                                               */
     int32_t precision;         /* cute_precision                                          */
-    float min_reuse;           /* AUTO: panels with nnz/activeCols below this go to ROWS; <=0: default */
+    float min_reuse;           /* AUTO: panels with fewer nonzeros per B row the MFMA side would fetch go to ROWS; <=0: default (1.25) */
     uint32_t slots;            /* resident work items assumed by the partition; 0: derive from device */
     uint32_t max_chunk_blocks; /* upper bound on blocks per work item; 0: none            */
     uint32_t brick_groups;     /* 16-lane column groups per lane in the brick kernel (1 or 2); 0: default */
     uint32_t pipeline;         /* brick kernel variant: 1 rolling, 2 pipelined; 0: default (rolling)             */
-    uint32_t mfma_shape;       /* MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists; 0: default (quad lists)     */
+    uint32_t mfma_shape;       /* MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists; 0: chosen per matrix (list slots per brick) */
     uint32_t max_row_nnz;      /* AUTO: panels holding a row longer than this stay on the brick kernel; 0: default  */
     uint32_t reserved[3];
 } cute_tunables;
@@ -324,7 +324,7 @@ typedef struct cute_plan_info {
     uint32_t N;
     uint32_t slabWidth;        /* columns of C per work item                              */
     uint32_t numSlabs;
-    uint32_t numChunks;        /* brick-kernel work items along the panel axis            */
+    uint32_t numChunks;        /* MFMA-kernel work items along the panel axis             */
     uint32_t numAtomicChunks;  /* of which are pieces of cut panels (partial tiles, added up by a second kernel; the name dates from atomics) */
     uint32_t numBrickPanels, numRowPanelsSparse, numEmptyPanels;
     uint32_t slots;
