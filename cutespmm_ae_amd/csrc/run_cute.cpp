@@ -45,6 +45,7 @@ int main(int argc, char **argv)
     }
     std::vector<unsigned> widths = {32, 128, 512};
     int iters = 20;
+    double ramp_ms = 30.0;     // launches before anything is timed: the GPU needs some milliseconds of work to reach its steady clocks
     bool keep_values = false, check = true;
     std::string cache_file;
     for (int i = 2; i < argc; ++i) {
@@ -53,6 +54,7 @@ int main(int argc, char **argv)
             widths.clear();
             for (char *tok = std::strtok(argv[++i], ","); tok; tok = std::strtok(nullptr, ",")) widths.push_back(unsigned(std::atoi(tok)));
         } else if (a == "--iters" && i + 1 < argc) iters = std::max(1, std::atoi(argv[++i]));
+        else if (a == "--ramp-ms" && i + 1 < argc) ramp_ms = std::max(0.0, std::atof(argv[++i]));
         else if (a == "--keep-values") keep_values = true;
         else if (a == "--no-check") check = false;
         else if (a == "--cache" && i + 1 < argc) cache_file = argv[++i];
@@ -111,27 +113,44 @@ int main(int argc, char **argv)
                 throw cute::Error(CUTE_ERR_HIP, "hipMemcpy B");
             SPMM_TC spmm(M, K, N, hrpb);
             spmm.run(dB.p, dC.p);
-            // timed like the comparison path (spmm.cu:941-953): warm-up launches, then `iters`
-            // launches between one pair of events, divided by `iters`
-            for (int w = 0; w < 3; ++w) spmm.run(dB.p, dC.p);
-            hipEvent_t e0, e1;
-            if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) throw cute::Error(CUTE_ERR_HIP, "hipEventCreate");
-            (void)hipEventRecord(e0, nullptr);
-            for (int it = 0; it < iters; ++it) spmm.run(dB.p, dC.p);
-            (void)hipEventRecord(e1, nullptr);
-            float total_ms = 0.0f;
-            if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&total_ms, e0, e1) != hipSuccess)
-                throw cute::Error(CUTE_ERR_HIP, "timing");
-            (void)hipEventDestroy(e0);
-            (void)hipEventDestroy(e1);
-            const double t_ms = double(total_ms) / iters;
+            // timed like the comparison path (spmm.cu:941-953): warm-up launches, then `iters` launches
+            // between one pair of events, divided by `iters` -- after `ramp_ms` of the same launches, for
+            // both columns of the table alike
+            auto time_launches = [&](auto &&launch) {
+                const auto ramp_end = std::chrono::steady_clock::now() + std::chrono::duration<double, std::milli>(ramp_ms);
+                while (std::chrono::steady_clock::now() < ramp_end) {
+                    for (int w = 0; w < 20; ++w) launch();
+                    if (hipDeviceSynchronize() != hipSuccess) throw cute::Error(CUTE_ERR_HIP, "ramp");
+                }
+                for (int w = 0; w < 3; ++w) launch();
+                hipEvent_t e0, e1;
+                if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) throw cute::Error(CUTE_ERR_HIP, "hipEventCreate");
+                (void)hipEventRecord(e0, nullptr);
+                for (int it = 0; it < iters; ++it) launch();
+                (void)hipEventRecord(e1, nullptr);
+                float total_ms = 0.0f;
+                if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&total_ms, e0, e1) != hipSuccess)
+                    throw cute::Error(CUTE_ERR_HIP, "timing");
+                (void)hipEventDestroy(e0);
+                (void)hipEventDestroy(e1);
+                return double(total_ms) / iters;
+            };
+            const double t_ms = time_launches([&] { spmm.run(dB.p, dC.p); });
             double ref_metric = -1.0, back_err = -1.0, csr_ms = -1.0;
             if (check) {
                 c_host.resize(size_t(M) * N);
                 c_ref.assign(size_t(M) * N, 0.0f);
                 if (hipMemcpy(c_host.data(), dC.p, c_host.size() * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
                     throw cute::Error(CUTE_ERR_HIP, "hipMemcpy C");
-                csr_ms = GPU_CSR_cuSPARSE_NEW(hrpb.rowPtr, hrpb.cols, hrpb.vals, nnz, b.data(), c_ref.data(), M, K, N, 5);
+                (void)GPU_CSR_cuSPARSE_NEW(hrpb.rowPtr, hrpb.cols, hrpb.vals, nnz, b.data(), c_ref.data(), M, K, N, 1);
+                // the CSR kernel's time: same kernel on the uploaded CSR copy, same timing protocol as above
+                const uint32_t *dRowPtr = nullptr, *dCols = nullptr;
+                const float *dVals = nullptr;
+                cute::check(cute_hrpb_dev_csr(hrpb.device, &dRowPtr, &dCols, &dVals), "cute_hrpb_dev_csr");
+                DeviceBuffer dC2(size_t(M) * N);
+                csr_ms = time_launches([&] {
+                    cute::check(cute_csr_spmm_dev(2, dRowPtr, dCols, dVals, dB.p, dC2.p, M, N, nullptr), "cute_csr_spmm_dev");
+                });
                 ref_metric = check_gemm_correctness_coo(c_ref.data(), c_host.data(), M, N);
                 back_err = cute_backward_error(hrpb.rowPtr, hrpb.cols, hrpb.vals, b.data(), c_ref.data(), c_host.data(), M, N);
             }
