@@ -33,6 +33,7 @@ ABI_SYMBOLS = [
     "cute_blocked_ell_build", "cute_blocked_ell_to_dense", "cute_blocked_ell_release",
     "cute_blocked_ell_upload", "cute_blocked_ell_dev_free", "cute_blocked_ell_spmm",
     "cute_splitter_split", "cute_split_release", "cute_classify_blocks", "cute_sequential_spmm",
+    "cute_block_stats", "cute_anxs",
 ]
 
 u32p = C.POINTER(C.c_uint32)
@@ -206,6 +207,8 @@ def load_library():
     lib.cute_split_release.argtypes = [C.POINTER(cute_split)]
     lib.cute_classify_blocks.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_float, C.c_float,
                                          C.POINTER(C.POINTER(cute_block_class)), C.POINTER(C.c_int64)]
+    lib.cute_block_stats.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, f32p]
+    lib.cute_anxs.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32, f32p]
     lib.cute_sequential_spmm.restype = C.c_float
     lib.cute_sequential_spmm.argtypes = [C.POINTER(cute_csr_i32), C.POINTER(C.c_double), C.POINTER(C.c_double),
                                          C.POINTER(C.c_double), C.c_int32, C.c_int32, C.c_int32]
@@ -799,6 +802,24 @@ class Splitter:
     def get_num_light_elems(self): return self._c[4]
     def get_heavyMatrix(self): return self._heavy
     def get_lightMatrix(self): return self._light
+
+
+def GET_STATS(A_CSR, blocksize):
+    """gpu_kernels.cu:1049-1137 -> float32[4]: mean nnz per active row and per active column of the non-empty
+    blocksize^2 blocks, their number, their mean density."""
+    raw = A_CSR._raw()
+    stats = np.zeros(4, np.float32)
+    _check(load_library().cute_block_stats(C.byref(raw), int(blocksize), _ptr(stats, f32p)), "cute_block_stats")
+    return stats
+
+
+def GET_ANXS(A_CSR, blocksize, axis):
+    """gpu_kernels.cu:1139-1186: nonzeros per distinct column of a block row (axis true) or per distinct row of
+    a block column (axis false)."""
+    raw = A_CSR._raw()
+    v = C.c_float()
+    _check(load_library().cute_anxs(C.byref(raw), int(blocksize), 1 if axis else 0, C.byref(v)), "cute_anxs")
+    return float(v.value)
 
 
 def classify_blocks(A_CSR, BlockSize, deviation_threshold, underload_dominance):

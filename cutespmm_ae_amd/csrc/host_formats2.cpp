@@ -473,4 +473,123 @@ float cute_sequential_spmm(const cute_csr_i32 *a, const double *vals, const doub
     return std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
 }
 
+// GET_STATS, gpu_kernels.cu:1049-1137.  The reference keys its hash maps with r_blk * (ncols / blocksize) + c_blk
+// (:1064-1067); when blocksize does not divide ncols the last block column of block row i therefore shares its key
+// with block (i + 1, 0), and with ncols < blocksize every block shares key 0.  Both are reproduced: the two
+// blocks count as one, their rows and columns (disjoint sets) add.  Terms are added in key order, in float.
+int cute_block_stats(const cute_csr_i32 *a, int32_t blocksize, float *stats)
+{
+    if (!csr_ok(a) || !stats || blocksize <= 0) return CUTE_ERR_ARG;
+    const int bs = blocksize, nbr = (a->nrows + bs - 1) / bs;
+    const uint64_t per_row = uint64_t(a->ncols) / uint64_t(bs);
+    if ((uint64_t(nbr) + 1) * per_row + per_row >= (uint64_t(1) << 32)) return CUTE_ERR_SHAPE;   // 32-bit keys would wrap
+    struct Blk { int bc, nnz, rows, cols; };
+    std::vector<std::vector<Blk>> per{static_cast<size_t>(nbr)};
+    parallel_ranges(uint64_t(nbr), 8, [&](uint64_t bb, uint64_t be, unsigned) {
+        std::vector<std::pair<int, int>> ent;          // (column, row inside the block row)
+        std::vector<int> stamp(size_t(bs), -1);
+        for (uint64_t br = bb; br < be; ++br) {
+            ent.clear();
+            const int r0 = int(br) * bs, r1 = std::min(a->nrows, r0 + bs);
+            for (int r = r0; r < r1; ++r)
+                for (int e = a->rowPtr[r]; e < a->rowPtr[r + 1]; ++e) ent.emplace_back(a->cols[e], r - r0);
+            std::sort(ent.begin(), ent.end());
+            std::fill(stamp.begin(), stamp.end(), -1);
+            std::vector<Blk> &out = per[br];
+            for (size_t i = 0; i < ent.size();) {
+                const int bc = per_row ? ent[i].first / bs : 0;
+                Blk b{bc, 0, 0, 0};
+                size_t j = i;
+                for (; j < ent.size() && (per_row ? ent[j].first / bs : 0) == bc; ++j) {
+                    b.nnz++;
+                    if (j == i || ent[j].first != ent[j - 1].first) b.cols++;
+                    if (stamp[size_t(ent[j].second)] != int(out.size())) { stamp[size_t(ent[j].second)] = int(out.size()); b.rows++; }
+                }
+                out.push_back(b);
+                i = j;
+            }
+        }
+    });
+    float anrs = 0.0f, ancs = 0.0f, dens = 0.0f;
+    uint32_t blocks = 0;
+    auto emit = [&](const Blk &b) {
+        dens += float(b.nnz) / float(bs * bs);
+        anrs += float(b.nnz) / float(b.rows);
+        ancs += float(b.nnz) / float(b.cols);
+        ++blocks;
+    };
+    if (per_row == 0) {                       // every nonzero has key 0: one block, its columns need a union
+        Blk all{0, 0, 0, 0};
+        std::vector<char> seen(size_t(a->ncols), 0);
+        for (int br = 0; br < nbr; ++br)
+            for (const Blk &b : per[size_t(br)]) { all.nnz += b.nnz; all.rows += b.rows; }
+        for (int e = 0; e < a->rowPtr[a->nrows]; ++e)
+            if (!seen[size_t(a->cols[e])]) { seen[size_t(a->cols[e])] = 1; all.cols++; }
+        if (all.nnz) emit(all);
+    } else {
+        Blk carry{0, 0, 0, 0};                // block (br - 1, per_row): its key is that of block (br, 0)
+        for (int br = 0; br <= nbr; ++br) {
+            const std::vector<Blk> empty_row;
+            const std::vector<Blk> &row = br < nbr ? per[size_t(br)] : empty_row;
+            size_t first = 0;
+            if (carry.nnz) {
+                if (!row.empty() && row[0].bc == 0) {
+                    carry.nnz += row[0].nnz; carry.rows += row[0].rows; carry.cols += row[0].cols;
+                    first = 1;
+                }
+                emit(carry);
+                carry = Blk{0, 0, 0, 0};
+            }
+            for (size_t i = first; i < row.size(); ++i) {
+                if (uint64_t(row[i].bc) == per_row) carry = row[i];
+                else emit(row[i]);
+            }
+        }
+    }
+    stats[0] = anrs / float(blocks);
+    stats[1] = ancs / float(blocks);
+    stats[2] = float(blocks);
+    stats[3] = dens / float(blocks);
+    return CUTE_OK;
+}
+
+// GET_ANXS, gpu_kernels.cu:1139-1186: nonzeros per distinct (band, segment) pair.  axis != 0: bands are block
+// rows, segments columns (how often a fetched B row is reused inside a row panel); axis == 0: bands are block
+// columns, segments rows.
+int cute_anxs(const cute_csr_i32 *a, int32_t blocksize, int32_t axis, float *out)
+{
+    if (!csr_ok(a) || !out || blocksize <= 0) return CUTE_ERR_ARG;
+    const int bs = blocksize;
+    std::vector<int64_t> part(host_threads() + 1, 0);
+    if (axis) {
+        const int nbr = (a->nrows + bs - 1) / bs;
+        parallel_ranges(uint64_t(nbr), 8, [&](uint64_t bb, uint64_t be, unsigned t) {
+            std::vector<int> c;
+            int64_t n = 0;
+            for (uint64_t br = bb; br < be; ++br) {
+                const int r0 = int(br) * bs, r1 = std::min(a->nrows, r0 + bs);
+                c.assign(a->cols + a->rowPtr[r0], a->cols + a->rowPtr[r1]);
+                std::sort(c.begin(), c.end());
+                n += int64_t(std::unique(c.begin(), c.end()) - c.begin());
+            }
+            part[t] = n;
+        });
+    } else {
+        parallel_ranges(uint64_t(a->nrows), 256, [&](uint64_t rb, uint64_t re, unsigned t) {
+            std::vector<int> c;
+            int64_t n = 0;
+            for (uint64_t r = rb; r < re; ++r) {
+                c.clear();
+                for (int e = a->rowPtr[r]; e < a->rowPtr[r + 1]; ++e) c.push_back(a->cols[e] / bs);
+                std::sort(c.begin(), c.end());
+                n += int64_t(std::unique(c.begin(), c.end()) - c.begin());
+            }
+            part[t] = n;
+        });
+    }
+    const int64_t sum = std::accumulate(part.begin(), part.end(), int64_t(0));
+    *out = float(uint32_t(a->rowPtr[a->nrows])) / float(int(sum));      // (float)nnz / sum, :1185
+    return CUTE_OK;
+}
+
 }  // extern "C"

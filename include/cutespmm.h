@@ -275,6 +275,18 @@ typedef struct cute_block_class {  /* one non-empty blockSize^2 block, inc/prepr
 int cute_classify_blocks(const cute_csr_i32 *csr, int32_t blockSize, float deviation_threshold,
                          float underload_dominance, cute_block_class **out, int64_t *count);
 
+/* GET_STATS, gpu_kernels.cu:1049-1137, the features its split threshold is chosen from: over the non-empty
+ * blocksize^2 blocks, stats[0] = mean of nnz / distinct rows, stats[1] = mean of nnz / distinct columns,
+ * stats[2] = number of blocks, stats[3] = mean of nnz / blocksize^2.  Blocks are told apart by the reference's
+ * key r_blk * (ncols / blocksize) + c_blk, so with ncols not a multiple of blocksize the last block column
+ * counts into block (r_blk + 1, 0), as there.  The reference adds its float terms in hash-map order; here they
+ * are added in key order (results agree to float rounding, not bit for bit).  CUTE_ERR_SHAPE where the
+ * reference's 32-bit keys would wrap.  An empty matrix gives NaN means and 0 blocks, as there. */
+int cute_block_stats(const cute_csr_i32 *csr, int32_t blocksize, float stats[4]);
+/* GET_ANXS, gpu_kernels.cu:1139-1186: nnz / number of distinct (band, segment) pairs; axis != 0: bands are
+ * block rows and segments columns, axis == 0: bands are block columns and segments rows. */
+int cute_anxs(const cute_csr_i32 *csr, int32_t blocksize, int32_t axis, float *out);
+
 /* sequentioal_spmm, inc/SPMM.cuh:123-187: double-precision CPU CSR SpMM; returns ms. */
 float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, const double *B, double *C,
                            int32_t m, int32_t k, int32_t n);

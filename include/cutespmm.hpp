@@ -307,3 +307,16 @@ private:
     cute_split s_{};
     SparseCoo<float> *heavy_ = nullptr, *light_ = nullptr;
 };
+
+// Block statistics the reference's harness chooses its split threshold from (gpu_kernels.cu:1049-1186).
+inline void GET_STATS(CSR_Matrix<float> *A_CSR, uint32_t blocksize, std::vector<float> &stats)
+{
+    if (stats.size() < 4) stats.resize(4);
+    cute::check(cute_block_stats(&A_CSR->raw(), int32_t(blocksize), stats.data()), "GET_STATS");
+}
+inline float GET_ANXS(CSR_Matrix<float> *A_CSR, uint32_t blocksize, bool axis)
+{
+    float v = 0.0f;
+    cute::check(cute_anxs(&A_CSR->raw(), int32_t(blocksize), axis ? 1 : 0, &v), "GET_ANXS");
+    return v;
+}

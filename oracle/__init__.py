@@ -217,6 +217,23 @@ def classify(nnz, under, over, B, deviation_threshold, underload_dominance):
                                   C.c_float(underload_dominance)))
 
 
+def get_stats(nrows, ncols, rowPtr, cols, blocksize):
+    """GET_STATS (gpu_kernels.cu:1049-1137): [ANRS, ANCS, non-empty blocks, mean block density] as float32."""
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    out = np.zeros(4, np.float32)
+    lib().orc_get_stats(C.c_int(nrows), C.c_int(ncols), _p(rowPtr, C.c_int), _p(cols, C.c_int), C.c_int(blocksize),
+                        _p(out, C.c_float))
+    return out
+
+
+def get_anxs(nrows, rowPtr, cols, blocksize, axis):
+    """GET_ANXS (gpu_kernels.cu:1139-1186)."""
+    rowPtr, cols = _csr_i32(rowPtr, cols)
+    f = lib().orc_get_anxs
+    f.restype = C.c_float
+    return float(f(C.c_int(nrows), _p(rowPtr, C.c_int), _p(cols, C.c_int), C.c_int(blocksize), C.c_int(1 if axis else 0)))
+
+
 def spmm_csr_f64(rowPtr, cols, vals, B):
     rowPtr, cols = _csr_i32(rowPtr, cols)
     vals, B = np.ascontiguousarray(vals, np.float64), np.ascontiguousarray(B, np.float64)

@@ -15,6 +15,9 @@
  *                                   heavy + light = A, disjoint; brute-force tile counts
  *   orc_block_stats / orc_classify  hand-worked rows incl. the band-walk's start and end rules
  *   orc_spmm_csr_f64                float64 numpy product
+ *   orc_get_stats / orc_get_anxs    dense-matrix brute force in numpy (distinct rows, columns, nonzeros
+ *                                   per block and per band); closed forms (identity, full blocks,
+ *                                   a single row or column per block)
  */
 #include <stdint.h>
 #include <stdio.h>
@@ -278,4 +281,81 @@ void orc_spmm_csr_f64(int m, int n, const int *rowPtr, const int *cols, const do
             for (int e = rowPtr[row]; e < rowPtr[row + 1]; ++e) sum += vals[e] * B[(size_t)n * cols[e] + col];
             C[(size_t)n * row + col] = sum;
         }
+}
+
+/* ------------------------------------------------------------------ */
+/* GET_STATS and GET_ANXS, gpu_kernels.cu:1049-1186                    */
+/* ------------------------------------------------------------------ */
+typedef struct { unsigned key; int seg; } orc_keyseg;
+
+static int orc_keyseg_cmp(const void *a, const void *b)
+{
+    const orc_keyseg *x = (const orc_keyseg *)a, *y = (const orc_keyseg *)b;
+    if (x->key != y->key) return x->key < y->key ? -1 : 1;
+    if (x->seg != y->seg) return x->seg < y->seg ? -1 : 1;
+    return 0;
+}
+
+/* Per non-empty block (key r_blk * (ncols / blocksize) + c_blk in 32-bit unsigned arithmetic, :1064-1067, so
+ * block columns beyond ncols / blocksize alias into the next block row exactly as the reference's map keys do):
+ * nonzeros, distinct rows, distinct columns.  stats[0] = mean of nnz / rows, [1] = mean of nnz / columns,
+ * [2] = number of blocks, [3] = mean of nnz / blocksize^2 (:1108-1136).  The reference adds the float terms
+ * in hash-map order; here they are added in key order, every term rounded to float as there (:1123-1125). */
+void orc_get_stats(int nrows, int ncols, const int *rowPtr, const int *cols, int blocksize, float *stats)
+{
+    const int nnz = rowPtr[nrows];
+    const unsigned per_row = (unsigned)ncols / (unsigned)blocksize;
+    orc_keyseg *by_row = (orc_keyseg *)malloc(sizeof(orc_keyseg) * (size_t)(nnz + 1));
+    orc_keyseg *by_col = (orc_keyseg *)malloc(sizeof(orc_keyseg) * (size_t)(nnz + 1));
+    int n = 0;
+    for (int r = 0; r < nrows; ++r)
+        for (int e = rowPtr[r]; e < rowPtr[r + 1]; ++e, ++n) {
+            const unsigned key = (unsigned)(r / blocksize) * per_row + (unsigned)(cols[e] / blocksize);
+            by_row[n].key = key; by_row[n].seg = r;
+            by_col[n].key = key; by_col[n].seg = cols[e];
+        }
+    qsort(by_row, (size_t)n, sizeof(orc_keyseg), orc_keyseg_cmp);
+    qsort(by_col, (size_t)n, sizeof(orc_keyseg), orc_keyseg_cmp);
+    float anrs = 0.0f, ancs = 0.0f, dens = 0.0f;
+    unsigned blocks = 0;
+    for (int i = 0; i < n;) {
+        int j = i, rows = 0, ccount = 0;
+        while (j < n && by_row[j].key == by_row[i].key) {
+            if (j == i || by_row[j].seg != by_row[j - 1].seg) rows++;
+            if (j == i || by_col[j].seg != by_col[j - 1].seg) ccount++;   /* same key runs: both arrays sort by key first */
+            ++j;
+        }
+        const int cnt = j - i;
+        dens += (float)cnt / (float)(blocksize * blocksize);
+        anrs += (float)cnt / (float)rows;
+        ancs += (float)cnt / (float)ccount;
+        blocks++;
+        i = j;
+    }
+    free(by_row);
+    free(by_col);
+    stats[0] = anrs / (float)blocks;
+    stats[1] = ancs / (float)blocks;
+    stats[2] = (float)blocks;
+    stats[3] = dens / (float)blocks;
+}
+
+/* nnz / (sum over bands of the distinct segments in the band), :1139-1186: axis != 0 takes block rows as
+ * bands and columns as segments, axis == 0 block columns and rows. */
+float orc_get_anxs(int nrows, const int *rowPtr, const int *cols, int blocksize, int axis)
+{
+    const int nnz = rowPtr[nrows];
+    orc_keyseg *ks = (orc_keyseg *)malloc(sizeof(orc_keyseg) * (size_t)(nnz + 1));
+    int n = 0;
+    for (int r = 0; r < nrows; ++r)
+        for (int e = rowPtr[r]; e < rowPtr[r + 1]; ++e, ++n) {
+            ks[n].key = (unsigned)(axis ? r / blocksize : cols[e] / blocksize);
+            ks[n].seg = axis ? cols[e] : r;
+        }
+    qsort(ks, (size_t)n, sizeof(orc_keyseg), orc_keyseg_cmp);
+    int sum = 0;
+    for (int i = 0; i < n; ++i)
+        if (i == 0 || ks[i].key != ks[i - 1].key || ks[i].seg != ks[i - 1].seg) sum++;
+    free(ks);
+    return (float)(unsigned)nnz / sum;      /* (float)nnz / sum with an int sum, :1185 */
 }

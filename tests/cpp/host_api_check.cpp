@@ -31,6 +31,10 @@ int main(int argc, char **argv)
                     hrpb.num_bricks, csr.BCSR_nblks, ell.get_ellColIdx_height(), ell.get_ellColIdx_width(), ell.get_num_blocks(),
                     split.get_total_tiles(), split.get_num_heavy_tiles(), split.get_num_heavy_elems(), split.get_num_light_tiles(),
                     split.get_num_light_elems(), diff, small.nnz, small.cols[0]);
+        std::vector<float> stats(4);
+        GET_STATS(&csr, 16, stats);
+        std::printf("stats=%.9g,%.9g,%.9g,%.9g anxs=%.9g,%.9g\n", stats[0], stats[1], stats[2], stats[3], GET_ANXS(&csr, 16, true),
+                    GET_ANXS(&csr, 16, false));
         if (argc > 2) {      // cache file: write, read back, compare every word
             hrpb.save(argv[2]);
             HRPB back(argv[2], /*upload=*/false);

@@ -4,6 +4,7 @@ import os
 import shutil
 import subprocess
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -25,3 +26,8 @@ def test_reference_style_host_program(cs, orc, tmp_path):
     assert (int(got["panels"]), int(got["blocks"]), int(got["words"])) == (h["numRowPanels"], h["numBlocks"], h["numWords"])
     assert got["bcsr"] == "8750" and got["tiles"] == "4325" and got["heavy"] == "1875/33800" and got["light"] == "2450/6200"
     assert got["densediff"] == "0" and got["grown"] == "2,1" and got["cache"] == "0"
+    dy, dx, _, r, c, v = orc.coo_read(mtx)
+    rp2, cl2, _ = orc.coo_to_csr(dy, r, c, v)
+    want = orc.get_stats(dy, dx, rp2, cl2, 16)
+    assert [np.float32(x) for x in got["stats"].split(",")] == want.tolist()
+    assert [np.float32(x) for x in got["anxs"].split(",")] == [np.float32(orc.get_anxs(dy, rp2, cl2, 16, a)) for a in (True, False)]

@@ -119,6 +119,50 @@ def test_oracle_double_spmm(orc):
     assert np.allclose(out, dense_from_csr(M, K, rp, cl, vl) @ B, rtol=1e-13, atol=1e-13)
 
 
+def _block_stats_brute(D, bs, ncols):
+    """Per key r_blk * (ncols // bs) + c_blk (gpu_kernels.cu:1064-1067): nonzeros, distinct rows, distinct columns."""
+    rows, cols = {}, {}
+    for r, c in zip(*np.nonzero(D)):
+        key = (r // bs) * (ncols // bs) + c // bs
+        rows.setdefault(key, []).append(r)
+        cols.setdefault(key, []).append(c)
+    nnz = np.array([len(rows[k]) for k in sorted(rows)], np.float64)
+    nr = np.array([len(set(rows[k])) for k in sorted(rows)], np.float64)
+    nc = np.array([len(set(cols[k])) for k in sorted(rows)], np.float64)
+    return np.array([(nnz / nr).mean(), (nnz / nc).mean(), len(nnz), (nnz / (bs * bs)).mean()])
+
+
+def test_oracle_get_stats_and_anxs(orc):
+    # closed forms.  Identity: every diagonal block holds bs nonzeros in bs rows and bs columns.
+    n, bs = 64, 16
+    rp, cl = np.arange(n + 1, dtype=np.int32), np.arange(n, dtype=np.int32)
+    assert orc.get_stats(n, n, rp, cl, bs).tolist() == [1.0, 1.0, 4.0, np.float32(1 / 16)]
+    assert orc.get_anxs(n, rp, cl, bs, True) == 1.0 and orc.get_anxs(n, rp, cl, bs, False) == 1.0
+    # all ones, 32 x 48: 6 full blocks; each block row holds 48 distinct columns, each block column 32 distinct rows
+    rp, cl = np.arange(33, dtype=np.int32) * 48, np.tile(np.arange(48, dtype=np.int32), 32)
+    assert orc.get_stats(32, 48, rp, cl, bs).tolist() == [16.0, 16.0, 6.0, 1.0]
+    assert orc.get_anxs(32, rp, cl, bs, True) == np.float32(32 * 48) / np.float32(2 * 48)
+    assert orc.get_anxs(32, rp, cl, bs, False) == np.float32(32 * 48) / np.float32(3 * 32)
+    # only the first row of every block row is full: 16 nonzeros in one row and 16 columns per block
+    rp = np.zeros(33, np.int32)
+    rp[1:17], rp[17:] = 48, 96
+    cl = np.tile(np.arange(48, dtype=np.int32), 2)
+    assert orc.get_stats(32, 48, rp, cl, bs).tolist() == [16.0, 1.0, 6.0, np.float32(1 / 16)]
+    # dense-matrix brute force, also where the block size does not divide the column count (the last block
+    # column then counts into the next block row's first block) and where it exceeds it (one block in all)
+    for seed, M, K, b, dens in [(50, 64, 96, 16, 0.05), (51, 48, 64, 8, 0.3), (52, 70, 90, 16, 0.08), (53, 40, 12, 16, 0.3),
+                                (54, 33, 50, 7, 0.15)]:
+        M, K, rp, cl, vl = _csr_case(seed, M, K, dens)
+        D = dense_from_csr(M, K, rp, cl, np.ones_like(vl))
+        want = _block_stats_brute(D, b, K)
+        got = orc.get_stats(M, K, rp, cl, b)
+        assert got[2] == want[2] and np.allclose(got, want, rtol=2e-6, atol=0)
+        per_band_cols = sum(int(np.any(D[i:i + b], axis=0).sum()) for i in range(0, M, b))
+        per_band_rows = sum(int(np.any(D[:, j:j + b], axis=1).sum()) for j in range(0, K, b))
+        assert orc.get_anxs(M, rp, cl, b, True) == np.float32(len(cl)) / np.float32(per_band_cols)
+        assert orc.get_anxs(M, rp, cl, b, False) == np.float32(len(cl)) / np.float32(per_band_rows)
+
+
 # ---------------------------------------------------------------- product against oracle
 def test_product_coo_and_csr_equal_oracle(cs, orc, tmp_path):
     coo = cs.SparseCoo(G67)
@@ -192,3 +236,28 @@ def test_product_double_spmm_equals_oracle(cs, orc):
     B = np.random.default_rng(1).standard_normal((K, 7))
     out, ms = csr.sequentioal_spmm(B)
     assert ms >= 0 and (out == orc.spmm_csr_f64(rp, cl, vl.astype(np.float64), B)).all()
+
+
+def test_product_block_statistics_equal_oracle(cs, orc):
+    cases = [(60, 64, 96, 16, 0.05), (61, 48, 64, 8, 0.3), (62, 70, 90, 16, 0.08), (63, 40, 12, 16, 0.3), (64, 33, 50, 7, 0.15),
+             (65, 200, 333, 32, 0.02), (66, 16, 16, 1, 0.5)]
+    for seed, M, K, b, dens in cases:
+        M, K, rp, cl, vl = _csr_case(seed, M, K, dens)
+        csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp, cols=cl, values=vl)
+        assert cs.GET_STATS(csr, b).tolist() == orc.get_stats(M, K, rp, cl, b).tolist()      # same order of additions
+        for axis in (True, False):
+            assert np.float32(cs.GET_ANXS(csr, b, axis)) == np.float32(orc.get_anxs(M, rp, cl, b, axis))
+    coo = cs.SparseCoo(G67)
+    csr = cs.CSR_Matrix(coo)
+    for b in (16, 32):
+        assert cs.GET_STATS(csr, b).tolist() == orc.get_stats(csr.nrows, csr.ncols, csr.rowPtr, csr.cols, b).tolist()
+        assert np.float32(cs.GET_ANXS(csr, b, True)) == np.float32(orc.get_anxs(csr.nrows, csr.rowPtr, csr.cols, b, True))
+    # 16x16 blocks of G67 hold 4 325 tiles, the count the splitter reports for the same tiling
+    assert cs.GET_STATS(csr, 16)[2] == 4325
+    empty = cs.CSR_Matrix(nrows=8, ncols=8, rowPtr=np.zeros(9, np.int32), cols=np.zeros(0, np.int32), values=np.zeros(0, np.float32))
+    st = cs.GET_STATS(empty, 4)
+    assert st[2] == 0 and np.isnan(st[0]) and np.isnan(cs.GET_ANXS(empty, 4, True))
+    with pytest.raises(cs.CuteError):
+        cs.GET_STATS(csr, 0)
+    with pytest.raises(cs.CuteError):
+        cs.GET_ANXS(csr, -1, True)
