@@ -186,6 +186,49 @@ def test_split_panels_add_up(cs, orc, torch_cuda):
             assert (dC.cpu().numpy() == first).all()
 
 
+def test_work_items_dealt_by_length(cs, orc, torch_cuda):
+    """The order in which the MFMA work items are listed decides where they run, not what they compute: panel
+    order, the planner's choice and a forced deal give the same bits, with panels of very different lengths,
+    with cut panels (partial tiles) among them, for one and for several column slabs, alone and fused with rows."""
+    rng = np.random.default_rng(21)
+    M, K = 4096, 4096
+    lengths = rng.integers(1, 40, M // 16)
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 700 if r in (40, 2000) else int(lengths[r // 16]))
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for N in (32, 128, 200):
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        for kw in (dict(path=cs.PATH_BRICK, mfma_shape=1), dict(path=cs.PATH_BRICK, mfma_shape=2), dict()):
+            outs = {}
+            for order in (1, 0, 2):
+                outs[order], plan = _run(cs, torch_cuda, h, B, chunk_order=order, **kw)
+                assert plan.info["dealtChunks"] == (0 if order == 1 else 1 if order == 2 else plan.info["dealtChunks"])
+                if order == 1 and "path" in kw:
+                    assert plan.info["numAtomicChunks"] > 0
+            assert cs.backward_error(rp, cl, vl, B, ref, outs[1]) <= BERR, (N, kw)
+            assert (outs[0] == outs[1]).all() and (outs[2] == outs[1]).all(), (N, kw)
+    # several work items per SIMD, of very different lengths, all on the device at once: the planner deals them by itself
+    M3, K3 = 32768, 2048
+    lengths = rng.integers(1, 24, M3 // 16)
+    rp3, cl3, vl3 = random_csr(rng, M3, K3, row_nnz=lambda r: int(lengths[r // 16]))
+    h3 = cs.HRPB(M3, K3, rp3, cl3, vl3)
+    B3 = rng.standard_normal((K3, 64)).astype(np.float32)
+    ref3 = orc.spmm_csr(rp3, cl3, vl3, B3)
+    for shape in (1, 2):
+        out, plan = _run(cs, torch_cuda, h3, B3, path=cs.PATH_BRICK, mfma_shape=shape)
+        assert plan.info["dealtChunks"] == 1 and plan.info["numChunks"] >= 2048
+        assert cs.backward_error(rp3, cl3, vl3, B3, ref3, out) <= BERR
+        same, plan = _run(cs, torch_cuda, h3, B3, path=cs.PATH_BRICK, mfma_shape=shape, chunk_order=1)
+        assert plan.info["dealtChunks"] == 0 and (same == out).all()
+    # equal panels stay in panel order
+    rp2, cl2, vl2 = random_csr(rng, 1024, 1024, row_nnz=lambda r: 8)
+    h2 = cs.HRPB(1024, 1024, rp2, cl2, vl2)
+    _, plan = _run(cs, torch_cuda, h2, rng.standard_normal((1024, 64)).astype(np.float32), path=cs.PATH_BRICK, mfma_shape=1)
+    assert plan.info["dealtChunks"] == 0
+    with pytest.raises(cs.CuteError):
+        cs.SPMM_TC(h2, 64, chunk_order=3)
+
+
 def test_csr_comparison_kernels(cs, orc, torch_cuda):
     torch = torch_cuda
     A = cs.gen_config(2, 1 / 16.0)
