@@ -82,6 +82,8 @@ def main():
     ap.add_argument("--path", choices=("auto", "mfma", "rows"), default="auto", help="kernel family (default: the planner's choice)")
     ap.add_argument("--mfma-shape", type=int, default=0, help="1: 16x16x4 brick kernel, 2: 4x4x1 quad kernel, 0: planner's choice")
     ap.add_argument("--pipeline", type=int, default=0, help="brick kernel variant: 1 rolling, 2 pipelined, 0: default")
+    ap.add_argument("--chunk-order", type=int, default=0,
+                    help="MFMA work items: 0 planner's choice, 1 panel order, 2 dealt to the SIMDs longest first")
     ap.add_argument("--graph", action="store_true",
                     help="record the K launches of the timed region into one HIP graph and replay it (launch-bound workloads)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -111,7 +113,7 @@ def main():
     dB = torch.from_numpy(B).cuda()
     dC = torch.empty((A.M, N), device="cuda")
     plan = cs.SPMM_TC(h, N, path={"auto": cs.PATH_AUTO, "mfma": cs.PATH_BRICK, "rows": cs.PATH_ROWS}[args.path],
-                      mfma_shape=args.mfma_shape, pipeline=args.pipeline)
+                      mfma_shape=args.mfma_shape, pipeline=args.pipeline, chunk_order=args.chunk_order)
     stream = torch.cuda.current_stream()
 
     ramp_end = time.perf_counter() + args.ramp_ms * 1e-3
@@ -174,7 +176,7 @@ def main():
                config=dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, blocks=h.numBlocks,
                            bricks=h.num_bricks, plan={k: plan.info[k] for k in
                                                       ("slabWidth", "numSlabs", "numChunks", "numAtomicChunks",
-                                                       "numBrickPanels", "numRowPanelsSparse")}),
+                                                       "numBrickPanels", "numRowPanelsSparse", "dealtChunks")}),
                roofline=roofline)
 
     ref = None
