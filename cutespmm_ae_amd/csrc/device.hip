@@ -389,6 +389,25 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // a brick work item spans 16*VEC columns: for narrow N take the narrowest tile that still covers N
     while (p->vec > 1 && 8u * uint32_t(p->vec) >= N) p->vec /= 2;
     p->ng = (p->vec == 4 && N >= 128) ? 2 : 1;   // two column groups per lane pay off from 128 columns on (measured)
+    // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
+    {
+        uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
+        while ((1u << logl) < need && logl < 6) ++logl;
+        p->rows_logl = int(logl);
+        const uint32_t w = (1u << logl) * p->rows_vec;
+        p->rows_slabs = (N + w - 1) / w;
+    }
+    // A mixed plan is one launch, and the two-group brick kernel holds only four wavefronts per SIMD: when its
+    // work-groups and the row blocks together exceed that, the row blocks queue behind each other and the launch
+    // takes as long as the two parts one after the other (bcsstk18, N = 128: 11.8 us against 5.1 + 6.5).  One
+    // column group per lane halves the registers and doubles the resident wavefronts; the same when the row blocks
+    // are the larger part of the launch anyway (ted_B, N = 128).
+    bool ng_for_mixed = false;
+    if (p->ng == 2 && t.brick_groups == 0 && n_brick && n_rows) {
+        const uint64_t row_blocks = (uint64_t(n_rows) * CUTE_TM * p->rows_slabs + (256u >> p->rows_logl) - 1) / (256u >> p->rows_logl);
+        const uint64_t groups = (uint64_t(n_brick) * ((N + 127u) / 128u) + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
+        if (row_blocks + groups > uint64_t(c.num_cus) * 4u || row_blocks >= groups) { p->ng = 1; ng_for_mixed = true; }
+    }
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
     if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
     // the rolling variant addresses B and the values with 32-bit byte offsets (24 x 24-bit product)
@@ -417,14 +436,6 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     const uint32_t slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
     const uint32_t num_slabs = (N + slab - 1) / slab;
     if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
-    // row kernel shape: lanes per row = smallest power of two covering N/VEC, at most 64
-    {
-        uint32_t need = (N + p->rows_vec - 1) / p->rows_vec, logl = 0;
-        while ((1u << logl) < need && logl < 6) ++logl;
-        p->rows_logl = int(logl);
-        const uint32_t w = (1u << logl) * p->rows_vec;
-        p->rows_slabs = (N + w - 1) / w;
-    }
 
     // chunk list for the brick kernel.  With t.slots set, the reference arithmetic
     // (spmm.cu:776-812) decides which panels are cut; its default there would cut every panel
@@ -557,7 +568,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // one launch for a mixed plan: the quad kernel with any row shape of 4-float lanes, the rolling brick
     // kernel in the shapes the planner itself picks for N (forced column groups fall back to two launches)
     const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
-    const bool brick_default_shape = p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
+    const bool brick_default_shape = ng_for_mixed || p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
     p->info.fusedLaunch = (rows_fusable && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
@@ -736,6 +747,7 @@ bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, hipS
     else if (v == 2 && g == 1 && l == 3) launch_brick_rows_as<2, 1, 3>(p, dB, dC, s, grid, per_xcd);
     else if (v == 4 && g == 1 && l == 4) launch_brick_rows_as<4, 1, 4>(p, dB, dC, s, grid, per_xcd);
     else if (v == 4 && g == 1 && l == 5) launch_brick_rows_as<4, 1, 5>(p, dB, dC, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 6) launch_brick_rows_as<4, 1, 6>(p, dB, dC, s, grid, per_xcd);
     else if (v == 4 && g == 2 && l == 5) launch_brick_rows_as<4, 2, 5>(p, dB, dC, s, grid, per_xcd);
     else if (v == 4 && g == 2 && l == 6) launch_brick_rows_as<4, 2, 6>(p, dB, dC, s, grid, per_xcd);
     else return false;
