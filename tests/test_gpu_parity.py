@@ -510,6 +510,70 @@ def test_planner_choices_on_varied_structures(cs, orc, torch_cuda, seed):
                 assert np.isfinite(out).all() and err <= BERR, (seed, kind, M, K, N, kw, err, plan.info)
 
 
+@pytest.mark.parametrize("K,N", [((1 << 24) + 64, 8), ((1 << 22) + 16, 264)])
+def test_dimensions_beyond_the_32_bit_offsets(cs, orc, torch_cuda, K, N):
+    """The rolling brick kernel and the quad kernel address B with 32-bit byte offsets from 24-bit products: with
+    2^24 columns or more, or a B of 4 GiB or more, the planner has to fall back to the pipelined brick kernel
+    (64-bit addresses, like the row kernel).  B lives on the device only; the oracle sees the rows that are used."""
+    torch = torch_cuda
+    rng = np.random.default_rng(31)
+    M = 256
+    pool = np.unique(np.concatenate([rng.integers(0, 1000, 200), rng.integers(K - 1000, K, 200), rng.integers(0, K, 400),
+                                     np.array([0, K - 1])]))
+    rowPtr, cols = np.zeros(M + 1, np.uint32), []
+    for r in range(M):
+        n = 0 if r in (7, 100) else 300 if r == 50 else int(rng.integers(1, 40))
+        cols.append(np.sort(rng.choice(len(pool), n, replace=False)))
+        rowPtr[r + 1] = rowPtr[r] + n
+    small_cols = np.concatenate(cols).astype(np.uint32)            # column ids inside the pool
+    vals = rng.standard_normal(len(small_cols)).astype(np.float32)
+    Bpool = rng.standard_normal((len(pool), N)).astype(np.float32)
+    ref = orc.spmm_csr(rowPtr, small_cols, vals, Bpool)
+    big_cols = pool[small_cols].astype(np.uint32)
+    assert big_cols.max() == K - 1
+    h = cs.HRPB(M, K, rowPtr, big_cols, vals)
+    dB = torch.zeros((K, N), device="cuda")
+    dB[torch.from_numpy(pool.astype(np.int64)).cuda()] = torch.from_numpy(Bpool).cuda()
+    for kw in (dict(path=cs.PATH_BRICK), dict(path=cs.PATH_BRICK, mfma_shape=2), dict(path=cs.PATH_BRICK, pipeline=1),
+               dict(path=cs.PATH_BRICK, max_chunk_blocks=2), dict(path=cs.PATH_ROWS), dict()):
+        plan = cs.SPMM_TC(h, N, **kw)
+        if plan.info["numChunks"]:
+            assert plan.info["mfmaShape"] == 1 and plan.info["pipeline"] == 2, (kw, plan.info)
+        dC = torch.full((M, N), float("nan"), device="cuda")
+        plan.run(dB, dC)
+        torch.cuda.synchronize()
+        out = dC.cpu().numpy()
+        assert np.isfinite(out).all() and cs.backward_error(rowPtr, small_cols, vals, Bpool, ref, out) <= BERR, kw
+
+
+def test_row_count_beyond_the_32_bit_offsets(cs, orc, torch_cuda):
+    """2^24 rows or more (almost all of them empty here): C is addressed with 64 bits, every row is still written."""
+    torch = torch_cuda
+    rng = np.random.default_rng(32)
+    M, K, N = (1 << 24) + 32, 1024, 4
+    busy = np.unique(np.concatenate([rng.integers(0, M, 3000), np.arange(M - 40, M), np.arange(0, 20)]))
+    counts = np.zeros(M, np.int64)
+    counts[busy] = rng.integers(1, 30, len(busy))
+    counts[M - 1] = 200
+    rowPtr = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    cols = np.concatenate([np.sort(rng.choice(K, int(c), replace=False)) for c in counts[busy]]).astype(np.uint32)
+    vals = rng.standard_normal(len(cols)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rowPtr, cols, vals, B)
+    h = cs.HRPB(M, K, rowPtr, cols, vals)
+    dB = torch.from_numpy(B).cuda()
+    for kw in (dict(), dict(path=cs.PATH_BRICK), dict(path=cs.PATH_ROWS)):
+        plan = cs.SPMM_TC(h, N, **kw)
+        if plan.info["numChunks"]:
+            assert plan.info["mfmaShape"] == 1 and plan.info["pipeline"] == 2, (kw, plan.info)
+        dC = torch.full((M, N), float("nan"), device="cuda")
+        plan.run(dB, dC)
+        torch.cuda.synchronize()
+        out = dC.cpu().numpy()
+        assert np.isfinite(out).all() and (out[counts == 0] == 0).all()
+        assert cs.backward_error(rowPtr, cols, vals, B, ref, out) <= BERR, kw
+
+
 def test_launches_can_be_captured_in_a_graph(cs, orc, torch_cuda):
     """cute_spmm_run only enqueues kernels (zeroing included), so a caller may capture it in a HIP
     graph: every replay, with B changed in place between replays, equals the eager result."""
