@@ -542,6 +542,8 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
     if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
     p->unitRows = CUTE_TM / upp;
+    // reduce_partials walks a tile along grid.y
+    if (rc == CUTE_OK && n_pieces && (uint64_t(CUTE_TM / upp) * N + 63u) / 64u > 65535u) rc = CUTE_ERR_SHAPE;
     if (rc == CUTE_OK && n_pieces) {
         // the kernels address the partial tiles like C, with 32-bit byte offsets
         const uint64_t bytes = uint64_t(n_pieces) * p->unitRows * N * sizeof(float);

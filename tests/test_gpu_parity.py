@@ -285,6 +285,15 @@ def test_plan_rejects_bad_arguments(cs, torch_cuda):
     plan = cs.SPMM_TC(h, 32)
     with pytest.raises(ValueError):
         plan.run(torch.zeros((32, 16), device="cuda"), torch.zeros((32, 32), device="cuda"))
+    # a cut panel's partial tiles are added up by a launch that walks a tile along grid.y: widths it cannot
+    # cover are refused when the plan is made (without cut panels the same width is accepted)
+    rp, cl, vl = random_csr(np.random.default_rng(2), 64, 4096, row_nnz=lambda r: 2000 if r == 3 else 2)
+    long_panel = cs.HRPB(64, 4096, rp, cl, vl)
+    assert cs.SPMM_TC(long_panel, 128, path=cs.PATH_BRICK).info["numAtomicChunks"] > 0
+    with pytest.raises(cs.CuteError) as e:
+        cs.SPMM_TC(long_panel, 300000, path=cs.PATH_BRICK)
+    assert e.value.status == -2
+    assert cs.SPMM_TC(h, 300000, path=cs.PATH_BRICK).info["numAtomicChunks"] == 0
 
 
 def test_driver_and_sweep_tool(cs, torch_cuda, tmp_path):
