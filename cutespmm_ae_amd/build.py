@@ -14,7 +14,12 @@ HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc
 
 # -packed-fp32-ops is switched off for device code: the compiler then never forms
 # v_pk_{add,mul,fma}_f32 from scalar float code.
-DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# -amdgpu-kernarg-preload-count: the first kernel arguments arrive in scalar registers when a wavefront starts
+# instead of being fetched by its first instructions (gfx940 and later; the compiler keeps a prologue that
+# fetches them for firmware without the feature).  Every wavefront's first dependent loads start that much
+# earlier: 2.6 % on the headline launch.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
           "-pthread"]
 
