@@ -100,6 +100,7 @@ struct cute_spmm_plan {
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
+    uint32_t *dHeads = nullptr;         // quad kernels: per chunk, the descriptor and the record of its first group
     // panels (or 4-row strips) cut into several chunks: each chunk stores a partial tile, reduce_partials adds them
     uint4 *dFixups = nullptr;           // {panel or strip, first piece, pieces, -}
     uint32_t numFixups = 0;
@@ -324,6 +325,7 @@ void cute_spmm_plan_free(cute_spmm_plan *p)
 {
     if (!p) return;
     (void)hipFree(p->dChunks);
+    (void)hipFree(p->dHeads);
     (void)hipFree(p->dFixups);
     (void)hipFree(p->dPartials);
     (void)hipFree(p->dRowList);
@@ -540,6 +542,15 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         p->info.dealtChunks = deal_chunks(chunks, num_slabs, uint32_t(c.num_cus) / cute_dev::kNumXcd,
                                           p->shape == 2 || p->ng == 1 ? 8u : 4u, t.chunk_order == 2) ? 1u : 0u;
     int rc = upload(&p->dChunks, chunks.data(), chunks.size());
+    if (rc == CUTE_OK && p->shape == 2 && !chunks.empty()) {
+        const uint64_t words = uint64_t(chunks.size()) * cute_dev::kQuadHeadWords;
+        if (hipMalloc(reinterpret_cast<void **>(&p->dHeads), words * sizeof(uint32_t)) != hipSuccess) rc = CUTE_ERR_NOMEM;
+        else {
+            hipLaunchKernelGGL(cute_dev::build_quad_heads, dim3(uint32_t((words + 255u) / 256u)), dim3(256), 0, nullptr, p->dChunks,
+                               uint32_t(chunks.size()), d->dQRecs, p->dHeads);
+            if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) rc = CUTE_ERR_HIP;
+        }
+    }
     if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
     p->unitRows = CUTE_TM / upp;
     // reduce_partials walks a tile along grid.y
@@ -778,7 +789,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
 #define CUTE_FUSED_LAUNCH(F, S, LL)                                                                                       \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
-                       grid.x, uint32_t(quad_blocks), p->dChunks, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,  \
+                       grid.x, uint32_t(quad_blocks), p->dHeads, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,   \
                        uint32_t(p->d->numQuadVals),                                                                  \
                        p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC,    \
                        p->dPartials, N)
@@ -799,7 +810,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
             rows_launched = true;
         } else {
 #define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
-    hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,        \
+    hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dHeads, p->info.numChunks, per_xcd,         \
                        p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, p->dPartials, N)
         if (full && strips) CUTE_QUAD_LAUNCH(true, true);
         else if (full) CUTE_QUAD_LAUNCH(true, false);

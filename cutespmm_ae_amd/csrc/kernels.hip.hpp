@@ -32,6 +32,7 @@ constexpr int kWavesPerGroup = 4;
 constexpr int kHdrWords = 32;
 constexpr int kNumXcd = 8;
 constexpr int kQuadRecordWords = 20;   // device record of one quad-list group: 16 columns, mask lo/hi, first value, pad
+constexpr int kQuadHeadWords = 32;     // quad kernels, per chunk: descriptor (4 words), first group's record, padding to 128 bytes
 
 // Work-groups are handed to the 8 XCDs round-robin; this maps the hardware id to a
 // logical id such that each XCD walks one contiguous range of logical ids (neighbouring
@@ -449,7 +450,7 @@ __device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32
 }
 
 template <bool FULL, bool STRIPS>
-__device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint4 *__restrict__ chunks,
+__device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint32_t *__restrict__ heads,
                                           uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
                                           const float *__restrict__ qvals, uint32_t zero_index,
                                           const float *__restrict__ B, float *__restrict__ C,
@@ -459,11 +460,18 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
     const uint32_t chunk = xcd_contiguous_id(block_x, groups_per_xcd) * kWavesPerGroup + wave;
     if (chunk >= num_chunks) return;
-    const uint4 ck = chunks[chunk];
-    const uint32_t g_end = __builtin_amdgcn_readfirstlane(ck.y);
-    const uint32_t panel = __builtin_amdgcn_readfirstlane(ck.z);
-    const uint32_t piece = __builtin_amdgcn_readfirstlane(ck.w);
-    uint32_t g = __builtin_amdgcn_readfirstlane(ck.x);
+    // One entry of kQuadHeadWords per chunk: its descriptor and, behind it, the record of its first group, so
+    // that the first B rows can be requested after one scalar fetch instead of two dependent ones.
+    const uint32_t *head = heads + size_t(chunk) * kQuadHeadWords;
+    uint32_t g = head[0];
+    const uint32_t g_end = head[1];
+    const uint32_t panel = head[2];
+    const uint32_t piece = head[3];
+    uint32_t head_rec[kQuadRecordWords];
+#pragma unroll
+    for (int p = 0; p < kQuadRecordWords; ++p) head_rec[p] = head[4 + p];
+    // one wait for the whole entry: the compiler would otherwise sink the later words to their first use
+    asm volatile("" ::"s"(head_rec[11]), "s"(head_rec[12]), "s"(head_rec[15]), "s"(head_rec[16]), "s"(head_rec[17]), "s"(head_rec[18]));
 
     const uint32_t n = block_y * kWaveSize + lane;
     const bool live = FULL || n < N;
@@ -495,7 +503,8 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
             const uint32_t off = (__builtin_amdgcn_inverse_ballot_w64(mask) ? rank : zero_index) * 4u;
             return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(qvals) + off);
         };
-        fetch_cols(ca, g);
+#pragma unroll
+        for (int p = 0; p < kQuadRecordWords; ++p) ca[p] = head_rec[p];
         fetch_cols(cb, g + 1);
         a0 = fetch_a(ca);
         a1 = fetch_a(cb);
@@ -578,13 +587,27 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
     }
 }
 
+// Fills the quad kernels' per-chunk entries from the chunk list and the group records (run once per plan).
+__global__ __launch_bounds__(256) void build_quad_heads(const uint4 *__restrict__ chunks, uint32_t num_chunks,
+                                                        const uint32_t *__restrict__ qrecs, uint32_t *__restrict__ heads)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_chunks * uint32_t(kQuadHeadWords)) return;
+    const uint32_t c = i / uint32_t(kQuadHeadWords), w = i % uint32_t(kQuadHeadWords);
+    const uint4 ck = chunks[c];
+    uint32_t v = 0;                                   // an empty chunk (a strip without pairs) keeps a zero record
+    if (w < 4u) v = w == 0 ? ck.x : w == 1 ? ck.y : w == 2 ? ck.z : ck.w;
+    else if (w < 4u + uint32_t(kQuadRecordWords) && ck.x < ck.y) v = qrecs[size_t(ck.x) * kQuadRecordWords + (w - 4u)];
+    heads[i] = v;
+}
+
 template <bool FULL, bool STRIPS>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
-    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
+    const uint32_t *__restrict__ heads, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs,
     const float *__restrict__ qvals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
     float *__restrict__ partials, uint32_t N)
 {
-    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, chunks, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C,
+    quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, heads, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C,
                             partials, N);
 }
 
@@ -849,7 +872,7 @@ __global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restri
 // contiguous ranges like the row kernel's own launch does.
 template <bool FULL, bool STRIPS, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
-    uint32_t quad_blocks_x, uint32_t quad_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
+    uint32_t quad_blocks_x, uint32_t quad_blocks, const uint32_t *__restrict__ heads, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
     const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
@@ -857,7 +880,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f
 {
     static_assert(kWaveSize * kWavesPerGroup == 256, "both bodies are written for 256-thread blocks");
     if (blockIdx.x < quad_blocks) {
-        quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, chunks, num_chunks, groups_per_xcd,
+        quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, heads, num_chunks, groups_per_xcd,
                                 qrecs, qvals, zero_index, B, C, partials, N);
     } else {   // quad_blocks is a multiple of the XCD count, so the XCD of a row block is (its index) % 8 as well
         uint32_t block_id;
