@@ -4,24 +4,28 @@
 // serialisation; the file layout below is this library's own.
 //
 //   offset  0  char[8]  "CUTEHRPB"
-//           8  u32      version (1)
+//           8  u32      version (2)
 //          12  u32      panel height (16)     16  u32  block width (16)     20  u32  brick width (4)
 //          24  u32 M    28 u32 K    32 u32 nnz    36 u32 numRowPanels    40 u32 numBlocks    44 u32 numBricks
 //          48  u64      numWords
-//          56  u64      FNV-1a 64 of every payload byte, in file order
+//          56  u64      FNV-1a 64 of the 56 header bytes before this field, then of every payload byte in file order
 //          64  payload: blockedRowPtr[P+1] u32, activeCols[nb*16] u32, sizePtr[nb+1] u64,
 //                       blocksData[numWords] u32, rowPtr[M+1] u32, cols[nnz] u32, vals[nnz] f32
 // Little-endian, no padding between arrays.  A reader rejects a wrong magic, version, tile shape,
-// length or checksum, and arrays whose end markers disagree with the header.
+// length or checksum, and -- because a checksum only guards against accidents -- every array whose
+// contents could send a later consumer out of bounds: pointers that do not ascend or whose end
+// markers disagree with the header, a column or active column >= K, a record offset that is not a
+// whole number of 128-word chunks or disagrees with the size the record itself states.
 #include "common.hpp"
 
+#include <cstddef>
 #include <cstdio>
 #include <cstring>
 
 namespace {
 
 constexpr char kMagic[8] = {'C', 'U', 'T', 'E', 'H', 'R', 'P', 'B'};
-constexpr uint32_t kVersion = 1;
+constexpr uint32_t kVersion = 2;
 
 struct FileHeader {
     char magic[8];
@@ -39,6 +43,45 @@ uint64_t fnv1a(uint64_t h, const void *data, uint64_t n)
 }
 
 struct Piece { const void *ptr; uint64_t bytes; };
+
+constexpr uint64_t kFnvBasis = 0xcbf29ce484222325ull;
+constexpr size_t kHeaderSummed = offsetof(FileHeader, checksum);    // 56: everything in front of the checksum
+
+// What the consumers of a loaded matrix rely on (cute_hrpb_retile walks blocksData by sizePtr, the
+// device kernels index B by cols and activeCols, the planner walks rowPtr and blockedRowPtr).
+bool arrays_consistent(const FileHeader &fh, const uint32_t *brp, const uint32_t *acols, const uint64_t *sp,
+                       const uint32_t *stream, const uint32_t *rp, const uint32_t *cols)
+{
+    if (brp[0] != 0 || brp[fh.numRowPanels] != fh.numBlocks || sp[0] != 0 || sp[fh.numBlocks] != fh.numWords ||
+        rp[0] != 0 || rp[fh.M] != fh.nnz)
+        return false;
+    for (uint32_t r = 0; r < fh.M; ++r)
+        if (rp[r + 1] < rp[r] || rp[r + 1] > fh.nnz) return false;
+    for (uint32_t i = 0; i < fh.nnz; ++i)
+        if (cols[i] >= fh.K) return false;
+    for (uint32_t p = 0; p < fh.numRowPanels; ++p)
+        if (brp[p + 1] < brp[p] || brp[p + 1] > fh.numBlocks) return false;
+    for (uint64_t i = 0; i < uint64_t(fh.numBlocks) * CUTE_TK; ++i)
+        if (acols[i] >= fh.K) return false;
+    uint64_t bits = 0, bricks = 0;
+    for (uint32_t b = 0; b < fh.numBlocks; ++b) {
+        if (sp[b + 1] <= sp[b] || sp[b + 1] > fh.numWords) return false;
+        const uint64_t step = sp[b + 1] - sp[b];
+        if (step % CUTE_CHUNK_WORDS) return false;
+        const uint32_t *rec = stream + sp[b];
+        uint32_t nnz_blk = 0;
+        for (uint32_t j = 0; j < 4; ++j) {
+            uint64_t bm;
+            std::memcpy(&bm, rec + 28 + 2 * j, 8);
+            nnz_blk += uint32_t(__builtin_popcountll(bm));
+            bricks += bm != 0;
+        }
+        const uint64_t words = (((nnz_blk + 1u) / 2u) * 2u + CUTE_META_WORDS + CUTE_CHUNK_WORDS - 1u) / CUTE_CHUNK_WORDS;
+        if (words * CUTE_CHUNK_WORDS != step || rec[26] != words) return false;
+        bits += nnz_blk;
+    }
+    return bits == fh.nnz && bricks == fh.numBricks;
+}
 
 }  // namespace
 
@@ -59,7 +102,7 @@ int cute_hrpb_save(const cute_hrpb_host *h, const char *path)
         {h->sizePtr, (uint64_t(h->numBlocks) + 1) * 8},          {h->blocksData, h->numWords * 4},
         {h->rowPtr, (uint64_t(h->M) + 1) * 4},                   {h->cols, uint64_t(h->nnz) * 4},
         {h->vals, uint64_t(h->nnz) * 4}};
-    uint64_t sum = 0xcbf29ce484222325ull;
+    uint64_t sum = fnv1a(kFnvBasis, &fh, kHeaderSummed);
     for (const Piece &p : pieces) sum = fnv1a(sum, p.ptr, p.bytes);
     fh.checksum = sum;
     FILE *f = std::fopen(path, "wb");
@@ -105,21 +148,18 @@ int cute_hrpb_load(const char *path, cute_csr *csr, cute_hrpb_host *h)
         ok = ok && arr[i];
     }
     int rc = ok ? CUTE_OK : CUTE_ERR_NOMEM;
-    uint64_t sum = 0xcbf29ce484222325ull;
+    uint64_t sum = fnv1a(kFnvBasis, &fh, kHeaderSummed);
     for (int i = 0; i < 7 && rc == CUTE_OK; ++i) {
         if (bytes[i] && std::fread(arr[i], 1, bytes[i], f) != bytes[i]) rc = CUTE_ERR_FORMAT;
         else sum = fnv1a(sum, arr[i], bytes[i]);
     }
     std::fclose(f);
     if (rc == CUTE_OK && sum != fh.checksum) rc = CUTE_ERR_FORMAT;
-    if (rc == CUTE_OK) {
-        const uint32_t *brp = static_cast<const uint32_t *>(arr[0]);
-        const uint64_t *sp = static_cast<const uint64_t *>(arr[2]);
-        const uint32_t *rp = static_cast<const uint32_t *>(arr[4]);
-        if (brp[0] != 0 || brp[fh.numRowPanels] != fh.numBlocks || sp[0] != 0 || sp[fh.numBlocks] != fh.numWords ||
-            rp[0] != 0 || rp[fh.M] != fh.nnz)
-            rc = CUTE_ERR_FORMAT;
-    }
+    if (rc == CUTE_OK &&
+        !arrays_consistent(fh, static_cast<const uint32_t *>(arr[0]), static_cast<const uint32_t *>(arr[1]),
+                           static_cast<const uint64_t *>(arr[2]), static_cast<const uint32_t *>(arr[3]),
+                           static_cast<const uint32_t *>(arr[4]), static_cast<const uint32_t *>(arr[5])))
+        rc = CUTE_ERR_FORMAT;
     if (rc != CUTE_OK) {
         for (void *p : arr) std::free(p);
         return rc;

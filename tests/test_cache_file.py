@@ -56,7 +56,7 @@ def test_damaged_files_are_rejected(cs, tmp_path):
         assert e.value.status == status
 
     rejected(b"NOTAFILE" + good[8:])                               # magic
-    rejected(good[:8] + struct.pack("<I", 2) + good[12:])          # version
+    rejected(good[:8] + struct.pack("<I", 1) + good[12:])          # version
     rejected(good[:-1])                                            # truncated
     rejected(good + b"\0")                                         # trailing bytes
     rejected(good[:100] + bytes([good[100] ^ 1]) + good[101:])     # one flipped payload bit
@@ -65,3 +65,72 @@ def test_damaged_files_are_rejected(cs, tmp_path):
     with pytest.raises(cs.CuteError) as e:
         cs.HRPB.load(str(tmp_path / "missing.hrpb"))
     assert e.value.status == -1
+
+
+def _fnv1a(data):
+    h = 0xcbf29ce484222325
+    for b in data:
+        h = ((h ^ b) * 0x100000001b3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def _resealed(data):
+    """The same bytes with the checksum field recomputed, as a forger (not an accident) would leave them."""
+    return data[:56] + struct.pack("<Q", _fnv1a(data[:56] + data[64:])) + data[64:]
+
+
+def test_header_is_covered_by_the_checksum(cs, tmp_path):
+    rng = np.random.default_rng(7)
+    rp, cl, vl = random_csr(rng, 32, 64, density=0.2)
+    path = str(tmp_path / "a.hrpb")
+    cs.HRPB(32, 64, rp, cl, vl).save(path)
+    good = open(path, "rb").read()
+    assert _resealed(good) == good                                 # the test's idea of the checksum is the library's
+    for off, val in ((28, 48), (28, 80), (44, 1)):                 # K smaller, K larger, brick count
+        bad = good[:off] + struct.pack("<I", val) + good[off + 4:]
+        p = str(tmp_path / "bad.hrpb")
+        open(p, "wb").write(bad)
+        with pytest.raises(cs.CuteError) as e:
+            cs.HRPB.load(p)
+        assert e.value.status == -9
+
+
+def test_forged_contents_are_rejected(cs, tmp_path):
+    """A file whose checksum is right but whose arrays would send a consumer out of bounds."""
+    rng = np.random.default_rng(8)
+    M, K = 32, 64
+    rp, cl, vl = random_csr(rng, M, K, density=0.2)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    path = str(tmp_path / "a.hrpb")
+    h.save(path)
+    good = open(path, "rb").read()
+    nb, P, nnz, words = h.numBlocks, h.numRowPanels, h.numNNZ, h.numWords
+    off_brp = 64
+    off_act = off_brp + 4 * (P + 1)
+    off_sp = off_act + 4 * nb * 16
+    off_data = off_sp + 8 * (nb + 1)
+    off_rp = off_data + 4 * words
+    off_cols = off_rp + 4 * (M + 1)
+
+    def patched(off, fmt, val):
+        return _resealed(good[:off] + struct.pack(fmt, val) + good[off + struct.calcsize(fmt):])
+
+    assert cl.max() >= 48
+    cases = {
+        "K below the largest column": patched(28, "<I", 48),
+        "a column beyond K": patched(off_cols, "<I", K),
+        "an active column beyond K": patched(off_act + 4, "<I", K + 5),
+        "nnz in the header": patched(32, "<I", nnz - 1),
+        "row pointers that descend": patched(off_rp + 4 * 3, "<I", nnz + 7),
+        "panel pointers that descend": patched(off_brp + 4, "<I", nb + 1),
+        "a record offset off the chunk grid": patched(off_sp + 8, "<Q", 64),
+        "a record offset beyond the stream": patched(off_sp + 8, "<Q", words + 128),
+        "a record that states another size": patched(off_data + 4 * 26, "<I", 9),
+        "a bitmap with one more bit": patched(off_data + 4 * 28, "<I", 0xFFFFFFFF),
+    }
+    for what, data in cases.items():
+        p = str(tmp_path / "forged.hrpb")
+        open(p, "wb").write(data)
+        with pytest.raises(cs.CuteError) as e:
+            cs.HRPB.load(p)
+        assert e.value.status == -9, what
