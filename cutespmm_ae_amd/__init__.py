@@ -18,7 +18,8 @@ LIB_PATH = os.environ.get("CUTESPMM_LIBRARY") or os.path.join(_HERE, "libcutespm
 # every symbol declared in include/cutespmm.h
 ABI_SYMBOLS = [
     "cute_status_string", "cute_last_hip_error", "cute_free",
-    "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows",
+    "cute_mtx_read", "cute_csr_release", "cute_csr_sort_rows", "cute_csr_merge_duplicates", "cute_coo_merge_duplicates",
+    "cute_spmm_coo", "cute_offsets_fit",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
     "cute_quad_build", "cute_quad_fill", "cute_quad_build_strips", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
@@ -148,6 +149,9 @@ def load_library():
     lib.cute_mtx_read.argtypes = [C.c_char_p, C.c_int, C.POINTER(cute_csr)]
     lib.cute_csr_release.argtypes = [C.POINTER(cute_csr)]
     lib.cute_csr_sort_rows.argtypes = [C.POINTER(cute_csr)]
+    lib.cute_csr_merge_duplicates.argtypes = [C.POINTER(cute_csr)]
+    lib.cute_spmm_coo.argtypes = [u32p, u32p, f32p, f32p, f32p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32]
+    lib.cute_offsets_fit.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64]
     lib.cute_hrpb_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_hrpb_host)]
     lib.cute_hrpb_host_release.argtypes = [C.POINTER(cute_hrpb_host)]
     lib.cute_hrpb_retile.argtypes = [C.POINTER(cute_hrpb_host), C.POINTER(cute_hrpb_tiled)]
@@ -191,6 +195,7 @@ def load_library():
                                        C.c_int, C.c_int, f32p]
     lib.cute_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_size_t]
     lib.cute_coo_read.argtypes = [C.c_char_p, C.POINTER(cute_coo)]
+    lib.cute_coo_merge_duplicates.argtypes = [C.POINTER(cute_coo)]
     lib.cute_coo_save_mtx.argtypes = [C.POINTER(cute_coo), C.c_char_p]
     lib.cute_coo_release.argtypes = [C.POINTER(cute_coo)]
     lib.cute_coo_to_csr.argtypes = [C.POINTER(cute_coo), C.POINTER(cute_csr_i32)]
@@ -283,6 +288,13 @@ class CSR:
 
     def sort_rows(self):
         _check(load_library().cute_csr_sort_rows(C.byref(self._raw)), "cute_csr_sort_rows")
+        return self
+
+    def merge_duplicates(self):
+        """Sorts the rows and adds up entries that share a position (in file order); nnz shrinks."""
+        _check(load_library().cute_csr_merge_duplicates(C.byref(self._raw)), "cute_csr_merge_duplicates")
+        self.nnz = self._raw.nnz
+        self._attach()
         return self
 
 
@@ -608,6 +620,21 @@ def GPU_CSR_cuSPARSE_NEW(rowPtr, cols, vals, nnz, hB, hC, m, k, n, iters, alg=2)
 # --------------------------------------------------------------------------------------
 # metrics
 # --------------------------------------------------------------------------------------
+def spmm_coo(rows, cols, vals, B, M, K=None):
+    """``spmm_coo`` (inc.h:71-83) on the host: C[M,N] from COO arrays in array order, fp32."""
+    rows, cols, vals = _as(rows, np.uint32), _as(cols, np.uint32), _as(vals, np.float32)
+    B = _as(B, np.float32)
+    K = B.shape[0] if K is None else int(K)
+    out = np.empty((int(M), B.shape[1]), np.float32)
+    _check(load_library().cute_spmm_coo(_ptr(rows, u32p), _ptr(cols, u32p), _ptr(vals, f32p), _ptr(B, f32p),
+                                        _ptr(out, f32p), int(M), K, B.shape[1], len(rows)), "cute_spmm_coo")
+    return out
+
+
+def offsets_fit(M, K, N, num_vals=0, partial_rows=0):
+    return bool(load_library().cute_offsets_fit(int(M), int(K), int(N), int(num_vals), int(partial_rows)))
+
+
 def check_gemm_correctness_coo(C_ref, C_test, M=None, N=None):
     a, b = _as(C_ref, np.float32), _as(C_test, np.float32)
     M = a.shape[0] if M is None else M
@@ -665,6 +692,15 @@ class SparseCoo:
     def save_mtx(self, path):
         raw = self._raw()
         _check(load_library().cute_coo_save_mtx(C.byref(raw), os.fsencode(path)), "cute_coo_save_mtx")
+
+    def merge_duplicates(self):
+        """Adds up entries that share a position (file order); the arrays shrink."""
+        self.rows, self.cols, self.values = self.rows.copy(), self.cols.copy(), self.values.copy()
+        raw = self._raw()
+        _check(load_library().cute_coo_merge_duplicates(C.byref(raw)), "cute_coo_merge_duplicates")
+        self.nnz = raw.nnz
+        self.rows, self.cols, self.values = self.rows[:self.nnz], self.cols[:self.nnz], self.values[:self.nnz]
+        return self
 
 
 class CSR_Matrix:

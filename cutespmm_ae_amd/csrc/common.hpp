@@ -4,7 +4,9 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstdlib>
+#include <cctype>
 #include <cstring>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -69,6 +71,51 @@ inline uint64_t bitmap_to_canonical(uint64_t lane)
         out |= 1ull << ((b & 15u) * 4u + (b >> 4));
     }
     return out;
+}
+
+// The banner line of a MatrixMarket file, "%%MatrixMarket matrix <format> <field> <symmetry>" (case-insensitive).
+// The reference's readers only search that line for the substring "symmetric" (IO.cu:16,
+// inc/SparseCoo.hpp:113); the value-keeping readers of this library tokenise it.
+struct MmBanner {
+    bool present = false;      // the line starts with %%MatrixMarket
+    bool valid = false;        // object, format, field and symmetry are all known words
+    bool array = false;        // format: array (dense, column-major) instead of coordinate
+    int field = 0;             // 0 real, 1 integer, 2 pattern, 3 complex
+    int symmetry = 0;          // 0 general, 1 symmetric, 2 skew-symmetric, 3 hermitian
+};
+
+inline MmBanner parse_mm_banner(const char *b, const char *e)
+{
+    MmBanner r;
+    std::vector<std::string> tok;
+    const char *s = b;
+    while (s < e) {
+        while (s < e && (*s == ' ' || *s == '\t' || *s == '\r')) ++s;
+        const char *w = s;
+        while (s < e && *s != ' ' && *s != '\t' && *s != '\r') ++s;
+        if (s > w) {
+            std::string t(w, s);
+            for (char &ch : t) ch = char(std::tolower(static_cast<unsigned char>(ch)));
+            tok.push_back(t);
+        }
+    }
+    if (tok.empty() || tok[0] != "%%matrixmarket") return r;
+    r.present = true;
+    if (tok.size() != 5 || tok[1] != "matrix") return r;
+    if (tok[2] == "array") r.array = true;
+    else if (tok[2] != "coordinate") return r;
+    const char *fields[4] = {"real", "integer", "pattern", "complex"};
+    const char *syms[4] = {"general", "symmetric", "skew-symmetric", "hermitian"};
+    int f = -1, y = -1;
+    for (int i = 0; i < 4; ++i) {
+        if (tok[3] == fields[i]) f = i;
+        if (tok[4] == syms[i]) y = i;
+    }
+    if (f < 0 || y < 0 || (r.array && f == 2)) return r;     // a dense file cannot be a pattern
+    r.field = f;
+    r.symmetry = y;
+    r.valid = true;
+    return r;
 }
 
 // splitmix64: the counter-based generator behind every synthetic input.

@@ -413,9 +413,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (t.brick_groups == 1 || (t.brick_groups == 2 && p->vec == 4)) p->ng = int(t.brick_groups);
     if (t.pipeline > 2) { delete p; return CUTE_ERR_ARG; }
     // the rolling variant addresses B and the values with 32-bit byte offsets (24 x 24-bit product)
-    const bool offsets_fit = d->K < (1u << 24) && d->M < (1u << 24) && uint64_t(N) * 4u < (1u << 24) &&
-                             uint64_t(d->K) * N * 4u <= 0xffffffffull && uint64_t(d->M + 16u) * N * 4u <= 0xffffffffull &&
-                             (d->numVals + 64u) * 4u <= 0xffffffffull;
+    const bool offsets_fit = cute_offsets_fit(d->M, d->K, N, d->numVals, 0) == 1;
     p->pipeline = t.pipeline ? int(t.pipeline) : 1;
     if (p->pipeline == 1 && !offsets_fit) p->pipeline = 2;
     if (t.mfma_shape > 2) { delete p; return CUTE_ERR_ARG; }
@@ -435,78 +433,91 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         p->shape = slots < 8u * bricks ? 2 : 1;
     }
     if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
-    const uint32_t slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
-    const uint32_t num_slabs = (N + slab - 1) / slab;
-    if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
+    // The chunk list depends on the MFMA kernel (its work units are blocks or list groups).  It is built,
+    // and if the partial tiles of the cut panels then turn out to be more rows than the fast kernels'
+    // 24-bit row operand can address, built once more for the pipelined brick kernel, whose stores use
+    // 64-bit offsets.
+    uint32_t slab = 0, num_slabs = 0, upp = 1, slots = 0, n_pieces = 0;
+    std::vector<uint4> chunks, fixups;
+    for (int attempt = 0;; ++attempt) {
+        slab = p->shape == 2 ? 64u : 16u * p->vec * p->ng;   // the quad kernel: one column per lane
+        num_slabs = (N + slab - 1) / slab;
+        if (num_slabs > 65535u) { delete p; return CUTE_ERR_ARG; }   // slabs are the y dimension of the launch
 
-    // chunk list for the brick kernel.  With t.slots set, the reference arithmetic
-    // (spmm.cu:776-812) decides which panels are cut; its default there would cut every panel
-    // that is one block above the (floored) mean as soon as the device holds all work items
-    // at once, which is the normal case on 256 CUs.  The default policy therefore cuts only
-    // outliers: a panel is split when it is more than twice as long as the per-item share
-    // of the whole job (and at least 8 blocks), into pieces of about that share.
-    // work units along a panel: 16-column blocks for the brick kernel, groups for the quad kernel
-    const std::vector<uint32_t> &unit = p->shape == 2 ? d->qgp : d->brp;
-    // units per panel: 4 when the quad lists are kept per 4-row strip
-    const uint32_t upp = (p->shape == 2 && d->quadRows == 4) ? 4u : 1u;
-    const uint32_t num_units = d->P * upp;
-    const uint32_t resident = uint32_t(c.num_cus) * 4u * 8u;   // 4 SIMDs x 8 wavefronts per CU
-    const uint32_t slots = t.slots ? t.slots : resident;
-    std::vector<uint32_t> quads;
-    if (t.slots) {
-        int64_t n = cute_partition(num_units, unit.data(), num_slabs, slots, nullptr, 0);
-        if (n < 0) { delete p; return int(n); }
-        quads.resize(uint64_t(n) * 4);
-        cute_partition(num_units, unit.data(), num_slabs, slots, quads.data(), uint64_t(n));
-    } else {
-        uint64_t work = 0;
-        uint64_t busy = 0;
-        for (uint32_t q = 0; q < num_units; ++q)
-            if (!to_rows[q / upp] && unit[q + 1] != unit[q]) { work += unit[q + 1] - unit[q]; ++busy; }
-        const uint64_t mean = busy ? (work + busy - 1) / busy : 1;
-        const uint64_t share = (work * num_slabs + resident - 1) / resident;
-        // the mean only counts while it is short: a matrix whose few MFMA panels are all very long
-        // (a handful of dense rows) must still be cut, or one wavefront walks a whole panel alone
-        const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, std::min<uint64_t>(mean, 16)), 8));
-        for (uint32_t q = 0; q < num_units; ++q) {
-            const uint32_t s = unit[q], e = unit[q + 1];
-            if (s == e || to_rows[q / upp]) continue;
-            const uint32_t nblk = e - s;
-            if (nblk <= 2 * target) {
-                quads.insert(quads.end(), {s, e, q, 0u});
-                continue;
+        // chunk list for the brick kernel.  With t.slots set, the reference arithmetic
+        // (spmm.cu:776-812) decides which panels are cut; its default there would cut every panel
+        // that is one block above the (floored) mean as soon as the device holds all work items
+        // at once, which is the normal case on 256 CUs.  The default policy therefore cuts only
+        // outliers: a panel is split when it is more than twice as long as the per-item share
+        // of the whole job (and at least 8 blocks), into pieces of about that share.
+        // work units along a panel: 16-column blocks for the brick kernel, groups for the quad kernel
+        const std::vector<uint32_t> &unit = p->shape == 2 ? d->qgp : d->brp;
+        // units per panel: 4 when the quad lists are kept per 4-row strip
+        upp = (p->shape == 2 && d->quadRows == 4) ? 4u : 1u;
+        const uint32_t num_units = d->P * upp;
+        const uint32_t resident = uint32_t(c.num_cus) * 4u * 8u;   // 4 SIMDs x 8 wavefronts per CU
+        slots = t.slots ? t.slots : resident;
+        std::vector<uint32_t> quads;
+        if (t.slots) {
+            int64_t n = cute_partition(num_units, unit.data(), num_slabs, slots, nullptr, 0);
+            if (n < 0) { delete p; return int(n); }
+            quads.resize(uint64_t(n) * 4);
+            cute_partition(num_units, unit.data(), num_slabs, slots, quads.data(), uint64_t(n));
+        } else {
+            uint64_t work = 0;
+            uint64_t busy = 0;
+            for (uint32_t q = 0; q < num_units; ++q)
+                if (!to_rows[q / upp] && unit[q + 1] != unit[q]) { work += unit[q + 1] - unit[q]; ++busy; }
+            const uint64_t mean = busy ? (work + busy - 1) / busy : 1;
+            const uint64_t share = (work * num_slabs + resident - 1) / resident;
+            // the mean only counts while it is short: a matrix whose few MFMA panels are all very long
+            // (a handful of dense rows) must still be cut, or one wavefront walks a whole panel alone
+            const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, std::min<uint64_t>(mean, 16)), 8));
+            for (uint32_t q = 0; q < num_units; ++q) {
+                const uint32_t s = unit[q], e = unit[q + 1];
+                if (s == e || to_rows[q / upp]) continue;
+                const uint32_t nblk = e - s;
+                if (nblk <= 2 * target) {
+                    quads.insert(quads.end(), {s, e, q, 0u});
+                    continue;
+                }
+                const uint32_t pieces = (nblk + target - 1) / target;
+                const uint32_t step = (nblk + pieces - 1) / pieces;
+                for (uint32_t cs = s; cs < e; cs += step) quads.insert(quads.end(), {cs, std::min(e, cs + step), q, 1u});
             }
-            const uint32_t pieces = (nblk + target - 1) / target;
-            const uint32_t step = (nblk + pieces - 1) / pieces;
-            for (uint32_t cs = s; cs < e; cs += step) quads.insert(quads.end(), {cs, std::min(e, cs + step), q, 1u});
         }
-    }
-    // A chunk of a cut panel carries the 1-based number of its partial tile; the pieces of one panel are
-    // consecutive (panels ascend through the list), and one fixup entry per cut panel adds them up afterwards.
-    std::vector<uint4> chunks;
-    std::vector<uint4> fixups;
-    uint32_t n_pieces = 0;
-    for (size_t i = 0; i + 3 < quads.size(); i += 4) {
-        const uint32_t s = quads[i], e = quads[i + 1], pan = quads[i + 2];
-        uint32_t cut = quads[i + 3];
-        if (to_rows[pan / upp]) continue;
-        const uint32_t len = e - s;
-        const uint32_t cap = t.max_chunk_blocks ? t.max_chunk_blocks : len;
-        if (len > cap) cut = 1;                    // cut further than the partition asked for
-        const uint32_t step = std::min(cap, len);
-        for (uint32_t cs = s; cs < e; cs += step) {
-            if (cut) {
-                if (fixups.empty() || fixups.back().x != pan) fixups.push_back(make_uint4(pan, n_pieces, 0u, 0u));
-                fixups.back().z++;
-                ++n_pieces;
+        // A chunk of a cut panel carries the 1-based number of its partial tile; the pieces of one panel are
+        // consecutive (panels ascend through the list), and one fixup entry per cut panel adds them up afterwards.
+        chunks.clear();
+        fixups.clear();
+        n_pieces = 0;
+        for (size_t i = 0; i + 3 < quads.size(); i += 4) {
+            const uint32_t s = quads[i], e = quads[i + 1], pan = quads[i + 2];
+            uint32_t cut = quads[i + 3];
+            if (to_rows[pan / upp]) continue;
+            const uint32_t len = e - s;
+            const uint32_t cap = t.max_chunk_blocks ? t.max_chunk_blocks : len;
+            if (len > cap) cut = 1;                    // cut further than the partition asked for
+            const uint32_t step = std::min(cap, len);
+            for (uint32_t cs = s; cs < e; cs += step) {
+                if (cut) {
+                    if (fixups.empty() || fixups.back().x != pan) fixups.push_back(make_uint4(pan, n_pieces, 0u, 0u));
+                    fixups.back().z++;
+                    ++n_pieces;
+                }
+                chunks.push_back(make_uint4(cs, std::min(e, cs + step), pan, cut ? n_pieces : 0u));
             }
-            chunks.push_back(make_uint4(cs, std::min(e, cs + step), pan, cut ? n_pieces : 0u));
         }
+        // a strip without pairs inside an MFMA-routed panel still has to be written (as zeros): an empty chunk
+        if (upp > 1)
+            for (uint32_t q = 0; q < num_units; ++q)
+                if (unit[q] == unit[q + 1] && !to_rows[q / upp]) chunks.push_back(make_uint4(unit[q], unit[q], q, 0u));
+        const bool lean = p->shape == 2 || p->pipeline == 1;
+        if (!lean || !n_pieces || cute_offsets_fit(d->M, d->K, N, 0, uint64_t(n_pieces) * (CUTE_TM / upp)) == 1) break;
+        if (attempt || t.mfma_shape == 2 || t.pipeline == 1) { delete p; return CUTE_ERR_SHAPE; }   // the caller forced a fast kernel
+        p->shape = 1;
+        p->pipeline = 2;
     }
-    // a strip without pairs inside an MFMA-routed panel still has to be written (as zeros): an empty chunk
-    if (upp > 1)
-        for (uint32_t q = 0; q < num_units; ++q)
-            if (unit[q] == unit[q + 1] && !to_rows[q / upp]) chunks.push_back(make_uint4(unit[q], unit[q], q, 0u));
     std::vector<uint32_t> row_list;
     for (uint32_t q = 0; q < d->P; ++q)
         if (to_rows[q])
@@ -556,10 +567,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // reduce_partials walks a tile along grid.y
     if (rc == CUTE_OK && n_pieces && (uint64_t(CUTE_TM / upp) * N + 63u) / 64u > 65535u) rc = CUTE_ERR_SHAPE;
     if (rc == CUTE_OK && n_pieces) {
-        // the kernels address the partial tiles like C, with 32-bit byte offsets
+        // (the fast kernels address the partial tiles like C, with 32-bit byte offsets: checked where the chunks were made)
         const uint64_t bytes = uint64_t(n_pieces) * p->unitRows * N * sizeof(float);
-        if (bytes > 0xffffffffull) rc = CUTE_ERR_NOMEM;
-        else if (hipMalloc(reinterpret_cast<void **>(&p->dPartials), bytes) != hipSuccess) rc = CUTE_ERR_NOMEM;
+        if (hipMalloc(reinterpret_cast<void **>(&p->dPartials), bytes) != hipSuccess) rc = CUTE_ERR_NOMEM;
     }
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }

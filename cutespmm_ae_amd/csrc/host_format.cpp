@@ -90,6 +90,108 @@ inline int next_int(const char *&s, const char *e, long long &v)
 
 }  // namespace
 
+namespace {
+
+struct Triplet { uint32_t r, c; float v; };
+
+// The value-keeping reader: tokenises the banner, so that skew-symmetric files mirror with the
+// opposite sign, dense ("array") files are read, and fields this library has no arithmetic for
+// (complex, hermitian) are refused instead of silently losing their imaginary parts.  Entries
+// come out in file order, a mirrored entry right behind its original, exactly where the
+// reference's loader puts them (IO.cu:71-84).  A file without a banner is read the way the
+// reference reads every file: "symmetric" anywhere on the first line means mirror.
+int read_triplets(const char *begin, const char *end_, long long &m, long long &k, std::vector<Triplet> &out)
+{
+    LineCursor lc{begin, end_};
+    const char *b, *e;
+    if (!lc.next(b, e)) return CUTE_ERR_IO;
+    const MmBanner bn = parse_mm_banner(b, e);
+    bool mirror;
+    float mirror_sign = 1.0f;
+    if (bn.present) {
+        if (!bn.valid || bn.field == 3 || bn.symmetry == 3) return CUTE_ERR_FORMAT;
+        mirror = bn.symmetry != 0;
+        if (bn.symmetry == 2) mirror_sign = -1.0f;
+    } else {
+        mirror = std::string(b, e).find("symmetric") != std::string::npos;
+    }
+    bool have_size = false;
+    while (lc.next(b, e)) {
+        if (b < e && *b == '%') continue;
+        if (skip_ws(b, e) >= e) continue;
+        have_size = true;
+        break;
+    }
+    if (!have_size) return CUTE_ERR_IO;
+    const char *s = b;
+    if (next_int(s, e, m) != 1 || next_int(s, e, k) != 1 || m <= 0 || k <= 0) return CUTE_ERR_IO;
+    if (m > 0xFFFFFFF0ll || k > 0xFFFFFFF0ll) return CUTE_ERR_SHAPE;
+    if (mirror && bn.present && m != k) return CUTE_ERR_FORMAT;
+    auto push = [&](long long r, long long c, float v) {
+        out.push_back(Triplet{uint32_t(r - 1), uint32_t(c - 1), v});
+        if (mirror && r != c) out.push_back(Triplet{uint32_t(c - 1), uint32_t(r - 1), mirror_sign * v});
+    };
+    if (bn.array) {
+        // dense, column-major, one value per line; symmetric files hold the lower triangle with,
+        // skew-symmetric ones without the diagonal.  Zeros are not entries.
+        long long r = bn.symmetry == 2 ? 2 : 1, c = 1;
+        while (lc.next(b, e)) {
+            const char *w = skip_ws(b, e);
+            if (w >= e || *w == '%') continue;
+            if (c > k || r > m) return CUTE_ERR_FORMAT;            // more values than the header promises
+            char *endp = nullptr;
+            const double d = std::strtod(w, &endp);
+            if (endp == w) return CUTE_ERR_IO;
+            if (d != 0.0) push(r, c, float(d));
+            if (++r > m) { ++c; r = bn.symmetry == 0 ? 1 : bn.symmetry == 1 ? c : c + 1; }
+        }
+        const bool complete = bn.symmetry == 2 ? (c >= k) : (c == k + 1);
+        return complete ? CUTE_OK : CUTE_ERR_FORMAT;
+    }
+    while (lc.next(b, e)) {
+        long long r, c;
+        s = b;
+        const int g = next_int(s, e, r);
+        if (g == 0) continue;                                      // blank line
+        if (g < 0 || next_int(s, e, c) != 1) return CUTE_ERR_IO;
+        if (r < 1 || r > m || c < 1 || c > k) return CUTE_ERR_RANGE;
+        if (mirror && r != c && (c > m || r > k)) return CUTE_ERR_RANGE;
+        float v = 1.0f;
+        const char *w = skip_ws(s, e);
+        if (w < e) {
+            char *endp = nullptr;
+            const double d = std::strtod(w, &endp);                // the buffer is NUL-terminated
+            if (endp != w) v = static_cast<float>(d);
+        }
+        push(r, c, v);
+    }
+    return CUTE_OK;
+}
+
+int csr_from_triplets(long long m, long long k, const std::vector<Triplet> &t, cute_csr *out)
+{
+    if (t.size() > 0xFFFFFFFFull) return CUTE_ERR_SHAPE;
+    const uint32_t M = uint32_t((m - 1) / CUTE_TM + 1) * CUTE_TM;   // IO.cu:30
+    const uint32_t K = uint32_t((k - 1) / CUTE_TK + 1) * CUTE_TK;   // IO.cu:31
+    uint32_t *rowPtr = alloc_array<uint32_t>(uint64_t(M) + 1);
+    uint32_t *cols = alloc_array<uint32_t>(t.size());
+    float *vals = alloc_array<float>(t.size());
+    if (!rowPtr || !cols || !vals) { std::free(rowPtr); std::free(cols); std::free(vals); return CUTE_ERR_NOMEM; }
+    for (const Triplet &x : t) rowPtr[x.r + 1]++;
+    for (uint32_t i = 0; i < M; ++i) rowPtr[i + 1] += rowPtr[i];
+    std::vector<uint32_t> fill(M, 0u);
+    for (const Triplet &x : t) {
+        const uint32_t pos = rowPtr[x.r] + fill[x.r]++;
+        cols[pos] = x.c;
+        vals[pos] = x.v;
+    }
+    out->M = M; out->K = K; out->nnz = uint32_t(t.size());
+    out->rowPtr = rowPtr; out->cols = cols; out->vals = vals;
+    return CUTE_OK;
+}
+
+}  // namespace
+
 extern "C" int cute_mtx_read(const char *path, int keep_values, cute_csr *out)
 {
     if (!path || !out) return CUTE_ERR_ARG;
@@ -106,6 +208,14 @@ extern "C" int cute_mtx_read(const char *path, int keep_values, cute_csr *out)
     if (got != size_t(fsz)) return CUTE_ERR_IO;
     buf[got] = '\0';
 
+    if (keep_values) {
+        long long m = 0, k = 0;
+        std::vector<Triplet> t;
+        const int rc = read_triplets(buf.data(), buf.data() + got, m, k, t);
+        return rc == CUTE_OK ? csr_from_triplets(m, k, t, out) : rc;
+    }
+
+    // keep_values == 0: the reference's reader, quirk for quirk.
     LineCursor lc{buf.data(), buf.data() + got};
     const char *b, *e;
     if (!lc.next(b, e)) return CUTE_ERR_IO;
@@ -158,23 +268,14 @@ extern "C" int cute_mtx_read(const char *path, int keep_values, cute_csr *out)
         s = b;
         if (next_int(s, e, r) == 0) continue;
         next_int(s, e, c);
-        float v = 1.0f;                  // IO.cu:68
-        if (keep_values) {
-            const char *w = skip_ws(s, e);
-            if (w < e) {
-                char *endp = nullptr;
-                double d = std::strtod(w, &endp);   // buffer is NUL-terminated
-                if (endp != w) v = static_cast<float>(d);
-            }
-        }
-        uint32_t rr = uint32_t(r - 1), cc = uint32_t(c - 1);
+        const uint32_t rr = uint32_t(r - 1), cc = uint32_t(c - 1);
         uint32_t pos = rowPtr[rr] + fill[rr]++;
         cols[pos] = cc;
-        vals[pos] = v;
+        vals[pos] = 1.0f;                // IO.cu:68
         if (symmetric && rr != cc) {
             pos = rowPtr[cc] + fill[cc]++;
             cols[pos] = rr;
-            vals[pos] = v;
+            vals[pos] = 1.0f;            // IO.cu:81
         }
     }
     out->M = M;
@@ -183,6 +284,32 @@ extern "C" int cute_mtx_read(const char *path, int keep_values, cute_csr *out)
     out->rowPtr = rowPtr;
     out->cols = cols;
     out->vals = vals;
+    return CUTE_OK;
+}
+
+// Sorts every row by column and adds up entries that share a (row, column) position, in the order
+// the file held them; the arrays shrink in place and nnz follows.  For files that list an entry
+// more than once (assembly output): the format builder refuses duplicate columns.
+extern "C" int cute_csr_merge_duplicates(cute_csr *c)
+{
+    if (!c || !c->rowPtr) return CUTE_ERR_ARG;
+    std::vector<std::pair<uint32_t, float>> tmp;
+    uint32_t w = 0, row_start = 0;
+    for (uint32_t r = 0; r < c->M; ++r) {
+        const uint32_t s = row_start, e = c->rowPtr[r + 1];
+        row_start = e;
+        tmp.clear();
+        for (uint32_t i = s; i < e; ++i) tmp.emplace_back(c->cols[i], c->vals[i]);
+        std::stable_sort(tmp.begin(), tmp.end(),
+                         [](const std::pair<uint32_t, float> &a, const std::pair<uint32_t, float> &b) { return a.first < b.first; });
+        c->rowPtr[r] = w;
+        for (size_t i = 0; i < tmp.size(); ++i) {
+            if (i && tmp[i].first == tmp[i - 1].first) c->vals[w - 1] += tmp[i].second;
+            else { c->cols[w] = tmp[i].first; c->vals[w] = tmp[i].second; ++w; }
+        }
+    }
+    c->rowPtr[c->M] = w;
+    c->nnz = w;
     return CUTE_OK;
 }
 
@@ -557,6 +684,21 @@ extern "C" int cute_hrpb_untile(const cute_hrpb_tiled *t, cute_hrpb_host *out)
 // ---------------------------------------------------------------------------------
 // launch partition (spmm.cu:776-812)
 // ---------------------------------------------------------------------------------
+// The fast kernels (rolling brick kernel, quad kernels) form every B, C and value address as a 32-bit byte
+// offset from a scalar base, and the row part of it with a 24 x 24-bit multiply: row index times row pitch.
+// That holds while every row and column index and the row pitch in bytes stay below 2^24 and every array
+// below 4 GiB -- including the matrix of partial tiles that the pieces of cut panels are stored to, which has
+// the row pitch of C and `partial_rows` rows (pieces x rows per piece).
+extern "C" int cute_offsets_fit(uint32_t M, uint32_t K, uint32_t N, uint64_t num_vals, uint64_t partial_rows)
+{
+    const uint64_t lim24 = 1ull << 24, lim32 = 0xffffffffull;
+    const uint64_t pitch = uint64_t(N) * 4u;
+    return (K < lim24 && uint64_t(M) + 16u < lim24 && pitch < lim24 && uint64_t(K) * pitch <= lim32 &&
+            (uint64_t(M) + 16u) * pitch <= lim32 && (num_vals + 64u) * 4u <= lim32 && partial_rows < lim24 &&
+            partial_rows * pitch <= lim32)
+               ? 1 : 0;
+}
+
 extern "C" int64_t cute_partition(uint32_t P, const uint32_t *brp, uint32_t nbN, uint32_t slots,
                                   uint32_t *out4, uint64_t cap)
 {
@@ -593,6 +735,44 @@ extern "C" int64_t cute_partition(uint32_t P, const uint32_t *brp, uint32_t nbN,
 // ---------------------------------------------------------------------------------
 // metrics
 // ---------------------------------------------------------------------------------
+// CPU SpMM with the sums of inc.h:71-83: C = 0, then every nonzero in array order adds v * B[c,:] onto
+// C[r,:], product and sum rounded separately.  The reference forks its thread team inside the loop over
+// the nonzeros, once per nonzero; here the nonzeros are first grouped by row (a stable counting sort, so
+// each row still sees its nonzeros in array order) and the rows are shared out among the threads, which
+// gives every element of C the same sequence of additions, bit for bit, at one fork per call.
+#pragma clang fp contract(off)
+extern "C" int cute_spmm_coo(const uint32_t *rows, const uint32_t *cols, const float *vals, const float *B, float *C,
+                             uint32_t M, uint32_t K, uint32_t N, uint32_t NNZ)
+{
+    if (!B || !C || (NNZ && (!rows || !cols || !vals))) return CUTE_ERR_ARG;
+    if (N == 0) return CUTE_ERR_SHAPE;
+    for (uint32_t i = 0; i < NNZ; ++i)
+        if (rows[i] >= M || cols[i] >= K) return CUTE_ERR_RANGE;
+    std::vector<uint32_t> start(size_t(M) + 1, 0u), order(NNZ);
+    for (uint32_t i = 0; i < NNZ; ++i) start[rows[i] + 1]++;
+    for (uint32_t r = 0; r < M; ++r) start[r + 1] += start[r];
+    {
+        std::vector<uint32_t> fill(start.begin(), start.end() - 1);
+        for (uint32_t i = 0; i < NNZ; ++i) order[fill[rows[i]]++] = i;
+    }
+    parallel_ranges(M, 64, [&](uint64_t rb, uint64_t re, unsigned) {
+        for (uint64_t r = rb; r < re; ++r) {
+            float *c = C + r * N;
+            std::memset(c, 0, size_t(N) * sizeof(float));
+            for (uint32_t q = start[r]; q < start[r + 1]; ++q) {
+                const uint32_t i = order[q];
+                const float v = vals[i];
+                const float *b = B + size_t(cols[i]) * N;
+                for (uint32_t j = 0; j < N; ++j) {
+                    const float prod = v * b[j];
+                    c[j] += prod;
+                }
+            }
+        }
+    });
+    return CUTE_OK;
+}
+
 extern "C" float cute_check_gemm_correctness(const float *C_ref, const float *C_test, uint32_t M, uint32_t N)
 {
     const uint64_t total = uint64_t(M) * N;

@@ -95,7 +95,14 @@ int cute_coo_read(const char *path, cute_coo *out)
     LineCursor lc{buf.data(), buf.data() + buf.size() - 1};
     const char *b, *e;
     if (!lc.next(b, e)) return CUTE_ERR_IO;
-    const bool symmetric = std::string(b, e).find("symmetric") != std::string::npos;   // SparseCoo.hpp:113
+    // SparseCoo.hpp:113 searches the first line for "symmetric" and mirrors with the same value.  With a
+    // proper banner the line is tokenised instead: skew-symmetric files mirror with the opposite sign,
+    // dense ("array") files are read, complex and hermitian files are refused (the reference would keep
+    // their real parts and say nothing).
+    const MmBanner bn = parse_mm_banner(b, e);
+    if (bn.present && (!bn.valid || bn.field == 3 || bn.symmetry == 3)) return CUTE_ERR_FORMAT;
+    const bool symmetric = bn.present ? bn.symmetry != 0 : std::string(b, e).find("symmetric") != std::string::npos;
+    const float mirror_sign = (bn.present && bn.symmetry == 2) ? -1.0f : 1.0f;
     bool have = false;
     while (lc.next(b, e)) {                                                            // :119-125
         if (b < e && *b == '%') continue;
@@ -108,13 +115,33 @@ int cute_coo_read(const char *path, cute_coo *out)
         char *p = const_cast<char *>(b), *q;
         dy = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; p = q;
         dx = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; p = q;
-        hdr = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO;
+        if (!bn.array) { hdr = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; }
     }
     if (dy <= 0 || dx <= 0 || dy > 0x7FFFFFFF || dx > 0x7FFFFFFF || hdr < 0) return CUTE_ERR_SHAPE;
+    if (bn.present && symmetric && dy != dx) return CUTE_ERR_FORMAT;
     struct Pt { int r, c; float v; };
     std::vector<Pt> pts;
     pts.reserve(size_t(hdr) * (symmetric ? 2 : 1));
-    while (lc.next(b, e)) {                                                            // :130-150
+    if (bn.array) {
+        // column-major, one value per line; symmetric: lower triangle with, skew-symmetric without the diagonal
+        long long r = bn.symmetry == 2 ? 2 : 1, c = 1;
+        while (lc.next(b, e)) {
+            const char *w = b;
+            while (w < e && (*w == ' ' || *w == '\t' || *w == '\r')) ++w;
+            if (w >= e || *w == '%') continue;
+            if (c > dx || r > dy) return CUTE_ERR_FORMAT;
+            char *q;
+            const double d = std::strtod(w, &q);
+            if (q == w) return CUTE_ERR_IO;
+            if (d != 0.0) {
+                pts.push_back(Pt{int(r - 1), int(c - 1), float(d)});
+                if (symmetric && r != c) pts.push_back(Pt{int(c - 1), int(r - 1), mirror_sign * float(d)});
+            }
+            if (++r > dy) { ++c; r = bn.symmetry == 0 ? 1 : bn.symmetry == 1 ? c : c + 1; }
+        }
+        if (!(bn.symmetry == 2 ? c >= dx : c == dx + 1)) return CUTE_ERR_FORMAT;
+    }
+    while (!bn.array && lc.next(b, e)) {                                               // :130-150
         // tokens are taken from this line only (strto* would skip a newline as white space)
         auto skip = [&](char *s) { while (s < e && (*s == ' ' || *s == '\t' || *s == '\r')) ++s; return s; };
         char *p = skip(const_cast<char *>(b)), *q;
@@ -135,7 +162,7 @@ int cute_coo_read(const char *path, cute_coo *out)
         pts.push_back(Pt{int(x - 1), int(y - 1), float(v)});
         if (symmetric && x != y) {
             if (y > dy || x > dx) return CUTE_ERR_RANGE;
-            pts.push_back(Pt{int(y - 1), int(x - 1), float(v)});
+            pts.push_back(Pt{int(y - 1), int(x - 1), mirror_sign * float(v)});
         }
     }
     if (pts.size() > 0x7FFFFFFFull) return CUTE_ERR_SHAPE;
@@ -150,6 +177,33 @@ int cute_coo_read(const char *path, cute_coo *out)
     out->values = alloc_array<float>(pts.size());
     if (!out->rows || !out->cols || !out->values) { cute_coo_release(out); return CUTE_ERR_NOMEM; }
     for (size_t i = 0; i < pts.size(); ++i) { out->rows[i] = pts[i].r; out->cols[i] = pts[i].c; out->values[i] = pts[i].v; }
+    return CUTE_OK;
+}
+
+// Adds up entries that share a (row, column) position, in the order the array holds them (for a file
+// just read: file order), after a stable sort by (row, column); nnz shrinks.  The reference keeps
+// duplicates as they are (SparseCoo.hpp:130-152), and so does cute_coo_read.
+int cute_coo_merge_duplicates(cute_coo *c)
+{
+    if (!c || c->nnz < 0 || (c->nnz && (!c->rows || !c->cols || !c->values))) return CUTE_ERR_ARG;
+    const size_t n = size_t(c->nnz);
+    std::vector<int> order(n);
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [c](int a, int b) {
+        return c->rows[a] != c->rows[b] ? c->rows[a] < c->rows[b] : c->cols[a] < c->cols[b];
+    });
+    std::vector<int32_t> r(n), cl(n);
+    std::vector<float> v(n);
+    size_t w = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const int o = order[i];
+        if (w && r[w - 1] == c->rows[o] && cl[w - 1] == c->cols[o]) v[w - 1] += c->values[o];
+        else { r[w] = c->rows[o]; cl[w] = c->cols[o]; v[w] = c->values[o]; ++w; }
+    }
+    std::copy(r.begin(), r.begin() + w, c->rows);
+    std::copy(cl.begin(), cl.begin() + w, c->cols);
+    std::copy(v.begin(), v.begin() + w, c->values);
+    c->nnz = int32_t(w);
     return CUTE_OK;
 }
 

@@ -111,8 +111,8 @@ int main(int argc, char **argv)
             DeviceBuffer dB(size_t(K) * N), dC(size_t(M) * N);
             if (hipMemcpy(dB.p, b.data(), size_t(K) * N * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
                 throw cute::Error(CUTE_ERR_HIP, "hipMemcpy B");
-            SPMM_TC spmm(M, K, N, hrpb);
-            spmm.run(dB.p, dC.p);
+            SPMM_TC spmm(M, K, N, hrpb.blockedRowPtr);                                              // run.cu:45
+            spmm.run(hrpb.blocksDevice, dB.p, dC.p, hrpb.activeColsDevice, hrpb.sizePtrDevice);     // run.cu:46-50
             // timed like the comparison path (spmm.cu:941-953): warm-up launches, then `iters` launches
             // between one pair of events, divided by `iters` -- after `ramp_ms` of the same launches, for
             // both columns of the table alike

@@ -53,8 +53,13 @@ void cute_free(void *p);       /* releases any array returned by this library   
  * host: MatrixMarket -> CSR.                       Replaces MTX_READER (IO.cu:2-88).
  * M and K are rounded up to multiples of 16 (IO.cu:30-31); symmetric files are mirrored
  * (IO.cu:42-44,77-84); entries stay in file order inside a row (IO.cu:71-75).
- * keep_values == 0 reproduces the reference (every value 1.0f, IO.cu:68,81);
- * keep_values != 0 parses the third token (1.0 for pattern files).
+ * keep_values == 0 reproduces the reference, quirk for quirk: every value 1.0f (IO.cu:68,81),
+ * "symmetric" anywhere on the first line means mirror (IO.cu:16).
+ * keep_values != 0 is the tolerant reader: the banner "%%MatrixMarket matrix <format> <field>
+ * <symmetry>" is tokenised; values are parsed (1.0 for pattern files); skew-symmetric files are
+ * mirrored with the opposite sign; "array" (dense, column-major) files are read, zeros dropped;
+ * complex and hermitian files, and banners with unknown words, give CUTE_ERR_FORMAT.  A file
+ * without a banner is read as the reference would.  Entries keep the reference's order.
  * ---------------------------------------------------------------------------------- */
 typedef struct cute_csr {
     uint32_t M, K, nnz;
@@ -68,6 +73,10 @@ void cute_csr_release(cute_csr *csr);
 /* Sorts every row by column (stable w.r.t. values) so that it satisfies the HRPB
  * precondition; returns CUTE_ERR_UNSORTED if a row holds a duplicate column. */
 int cute_csr_sort_rows(cute_csr *csr);
+/* Same sort, and entries that share a (row, column) position are added up in file order; the
+ * arrays shrink in place and nnz follows.  No counterpart in the reference (IO.cu keeps
+ * duplicates, which HRPB's precondition, data.cu:204,256-258, then forbids). */
+int cute_csr_merge_duplicates(cute_csr *csr);
 
 /* ------------------------------------------------------------------------------------
  * host: CSR -> canonical HRPB.          Replaces HRPB::HRPB + DATASTRUCT (data.cu:80-335).
@@ -174,6 +183,11 @@ void cute_quad_release(cute_quad_lists *q);
  * ---------------------------------------------------------------------------------- */
 int64_t cute_partition(uint32_t numRowPanels, const uint32_t *blockedRowPtr, uint32_t nbN,
                        uint32_t slots, uint32_t *out4, uint64_t cap);
+/* 1 when the fast kernels' addressing (32-bit byte offsets, rows through a 24 x 24-bit multiply) covers a
+ * product of this size: M, K rows and columns, N columns of B and C, num_vals stored values, partial_rows
+ * rows of partial tiles (pieces of cut panels x rows per piece); else 0, and the planner takes the
+ * kernels with 64-bit offsets.  The limits stand where spmm.cu:11-101 has its per-N launch constants. */
+int cute_offsets_fit(uint32_t M, uint32_t K, uint32_t N, uint64_t num_vals, uint64_t partial_rows);
 
 /* ------------------------------------------------------------------------------------
  * host: result comparison.   Replaces check_gemm_correctness_coo (inc.h:84-109):
@@ -182,6 +196,11 @@ int64_t cute_partition(uint32_t numRowPanels, const uint32_t *blockedRowPtr, uin
  * max_ij |C_ref-C_test|_ij / sum_k |a_ik||b_kj| (0/0 counts as 0).
  * ---------------------------------------------------------------------------------- */
 float cute_check_gemm_correctness(const float *C_ref, const float *C_test, uint32_t M, uint32_t N);
+/* host: CPU SpMM.  Replaces spmm_coo (inc.h:71-83): C = 0, then every nonzero i in array order adds
+ * vals[i] * B[cols[i],:] onto C[rows[i],:] in fp32, product and sum rounded separately.  Same bits as
+ * that loop; the rows are shared out among the host threads instead of forking a team per nonzero. */
+int cute_spmm_coo(const uint32_t *rows, const uint32_t *cols, const float *vals, const float *B, float *C,
+                  uint32_t M, uint32_t K, uint32_t N, uint32_t NNZ);
 float cute_backward_error(const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
                           const float *B, const float *C_ref, const float *C_test,
                           uint32_t M, uint32_t N);
@@ -217,8 +236,12 @@ typedef struct cute_csr_i32 {      /* CSR_Matrix<float>, inc/CSR.hpp:42-51      
 } cute_csr_i32;
 
 /* SparseCoo<T>(path), inc/SparseCoo.hpp:91-157: keeps values (1.0 if absent), mirrors
- * symmetric files, sorts by (row, col). */
+ * symmetric files, sorts by (row, col).  The banner is tokenised as in cute_mtx_read with
+ * keep_values: skew-symmetric mirrors with the opposite sign, array files are read, complex and
+ * hermitian give CUTE_ERR_FORMAT (the reference searches the line for "symmetric" only, :113). */
 int cute_coo_read(const char *path, cute_coo *out);
+/* Adds up entries that share a position (after a stable sort by (row, col)); nnz shrinks. */
+int cute_coo_merge_duplicates(cute_coo *coo);
 /* save_mtx, inc/SparseCoo.hpp:263-285 ("real general", 1-based, one entry per line). */
 int cute_coo_save_mtx(const cute_coo *coo, const char *path);
 void cute_coo_release(cute_coo *coo);

@@ -2,11 +2,15 @@
 //
 // Same class names, public fields and call sequence as the reference's driver uses
 // (run.cu:11-62):   MTX_READER r(path);  HRPB hrpb(M, K, r.rowPtr, r.cols, r.vals);
-//                   SPMM_TC spmm(M, K, N, hrpb);  spmm.run(dB, dC);
+//                   SPMM_TC spmm(M, K, N, hrpb.blockedRowPtr);
+//                   spmm.run(hrpb.blocksDevice, dB, dC, hrpb.activeColsDevice, hrpb.sizePtrDevice);
+// (or the shorter forms SPMM_TC spmm(M, K, N, hrpb); spmm.run(dB, dC, stream);).
 // Differences, all deliberate: every object frees what it owns; errors throw
 // cute::Error instead of exit(-1) (inc.h:63-70) or a float-typed EXIT_FAILURE
 // (spmm.cu:841-859); HRPB checks its preconditions; C need not be zeroed by the caller.
 #pragma once
+#include <map>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 
@@ -22,6 +26,16 @@ struct Error : std::runtime_error {
           status(s) {}
 };
 inline void check(int s, const char *where) { if (s != CUTE_OK) throw Error(s, where); }
+
+// The reference's planner is constructed from the format's blockedRowPtr array alone (spmm.cu:276) and its
+// run() is handed three more device arrays of the same format (spmm.cu:823).  Here the device side of a
+// format is one handle, so every live HRPB is listed under the address of its blockedRowPtr array and the
+// reference-shaped SPMM_TC constructor finds the format -- and with it the handle -- from that pointer.
+struct HrpbRegistry {
+    std::mutex lock;
+    std::map<const unsigned int *, const void *> live;     // blockedRowPtr -> HRPB object
+    static HrpbRegistry &get() { static HrpbRegistry r; return r; }
+};
 
 }  // namespace cute
 
@@ -63,7 +77,12 @@ public:
     unsigned int *activeCols = nullptr;
     unsigned int numNNZ = 0;
     float block_density = 0.0f;       // nonzeros per slot of the non-empty bricks
-    cute_hrpb_dev *device = nullptr;  // stands for the four *Device pointers of data.cu:65-72
+    cute_hrpb_dev *device = nullptr;  // the device copy (both MFMA layouts and the CSR arrays)
+    // The four *Device fields of data.cu:65-72.  The device copy is not the canonical stream, so these are
+    // not addresses of such arrays: they are tokens (the handle above, retyped; null without a device copy)
+    // whose only use is to be passed to SPMM_TC::run as run.cu:46-50 does, which checks them.
+    unsigned int *blocksDevice = nullptr, *blockedRowPtrDevice = nullptr, *activeColsDevice = nullptr;
+    unsigned long long *sizePtrDevice = nullptr;
 
     HRPB(unsigned int M_, unsigned int K_, unsigned int *rowPtr_, unsigned int *cols_, float *vals_, bool upload = true)
         : cols(cols_), rowPtr(rowPtr_), vals(vals_), M(M_), K(K_), numRowPanels(M_ / CUTE_TM)
@@ -81,9 +100,33 @@ public:
         publish(upload);
     }
     void save(const char *cache_file) const { cute::check(cute_hrpb_save(&host_, cache_file), "HRPB save"); }
-    void freeDevice() { cute_hrpb_dev_free(device); device = nullptr; }   // data.cu:336-339
+    void freeDevice()                                                       // data.cu:336-339
+    {
+        cute_hrpb_dev_free(device);
+        device = nullptr;
+        blocksDevice = blockedRowPtrDevice = activeColsDevice = nullptr;
+        sizePtrDevice = nullptr;
+    }
     const cute_hrpb_host &host() const { return host_; }
-    ~HRPB() { freeDevice(); cute_hrpb_host_release(&host_); cute_csr_release(&owned_csr_); }
+    // The live format whose blockedRowPtr array this is, or null.
+    static const HRPB *find(const unsigned int *blockedRowPtr_)
+    {
+        cute::HrpbRegistry &r = cute::HrpbRegistry::get();
+        std::lock_guard<std::mutex> g(r.lock);
+        auto it = r.live.find(blockedRowPtr_);
+        return it == r.live.end() ? nullptr : static_cast<const HRPB *>(it->second);
+    }
+    ~HRPB()
+    {
+        {
+            cute::HrpbRegistry &r = cute::HrpbRegistry::get();
+            std::lock_guard<std::mutex> g(r.lock);
+            r.live.erase(blockedRowPtr);
+        }
+        freeDevice();
+        cute_hrpb_host_release(&host_);
+        cute_csr_release(&owned_csr_);
+    }
     HRPB(const HRPB &) = delete;
     HRPB &operator=(const HRPB &) = delete;
 
@@ -103,7 +146,12 @@ private:
         if (upload) {
             int rc = cute_hrpb_upload(&host_, &device);
             if (rc != CUTE_OK) { cute_hrpb_host_release(&host_); cute_csr_release(&owned_csr_); throw cute::Error(rc, "HRPB upload"); }
+            blocksDevice = blockedRowPtrDevice = activeColsDevice = reinterpret_cast<unsigned int *>(device);
+            sizePtrDevice = reinterpret_cast<unsigned long long *>(device);
         }
+        cute::HrpbRegistry &r = cute::HrpbRegistry::get();
+        std::lock_guard<std::mutex> g(r.lock);
+        r.live[blockedRowPtr] = this;
     }
 };
 
@@ -116,15 +164,31 @@ public:
     SPMM_TC(unsigned int M_, unsigned int K_, unsigned int N_, const HRPB &hrpb, const cute_tunables *tunables = nullptr)
         : M(M_), N(N_), K(K_)
     {
-        if (!hrpb.device) throw cute::Error(CUTE_ERR_ARG, "SPMM_TC: HRPB has no device copy");
-        cute::check(cute_spmm_plan_create(hrpb.device, N, tunables, &plan_), "SPMM_TC");
-        cute_spmm_plan_info(plan_, &info);
-        numRowPanelsSplit = info.numChunks;
+        create(hrpb, tunables);
+    }
+    // The reference's own signature (spmm.cu:276; call site run.cu:45): the format is found from its
+    // blockedRowPtr array, which must belong to a live HRPB object that has a device copy.
+    SPMM_TC(unsigned int M_, unsigned int K_, unsigned int N_, unsigned int *blockedRowPtr) : M(M_), N(N_), K(K_)
+    {
+        const HRPB *hrpb = HRPB::find(blockedRowPtr);
+        if (!hrpb) throw cute::Error(CUTE_ERR_ARG, "SPMM_TC: blockedRowPtr does not belong to a live HRPB");
+        if (hrpb->M != M || hrpb->K != K) throw cute::Error(CUTE_ERR_SHAPE, "SPMM_TC: M, K differ from the HRPB's");
+        create(*hrpb, nullptr);
     }
     // MatB [K x N], MatC [M x N]: device pointers; asynchronous on `stream`.
     void run(const float *MatB, float *MatC, void *stream = nullptr)
     {
         cute::check(cute_spmm_run(plan_, MatB, MatC, stream), "SPMM_TC::run");
+    }
+    // The reference's own signature (spmm.cu:823; call site run.cu:50), asynchronous on the default stream.
+    // The three format arguments must be the *Device fields of the HRPB this plan was made for; the plan
+    // already holds that format, so they are only checked.
+    void run(unsigned int *MatA, float *MatB, float *MatC, unsigned int *active_cols_vec, unsigned long long int *sizePtr)
+    {
+        const void *want = format_;
+        if (MatA != want || active_cols_vec != want || sizePtr != want)
+            throw cute::Error(CUTE_ERR_ARG, "SPMM_TC::run: MatA, active_cols_vec, sizePtr are not this plan's HRPB device fields");
+        run(MatB, MatC, nullptr);
     }
     cute_spmm_plan *plan() { return plan_; }
     ~SPMM_TC() { cute_spmm_plan_free(plan_); }
@@ -133,7 +197,23 @@ public:
 
 private:
     cute_spmm_plan *plan_ = nullptr;
+    const cute_hrpb_dev *format_ = nullptr;
+    void create(const HRPB &hrpb, const cute_tunables *tunables)
+    {
+        if (!hrpb.device) throw cute::Error(CUTE_ERR_ARG, "SPMM_TC: HRPB has no device copy");
+        cute::check(cute_spmm_plan_create(hrpb.device, N, tunables, &plan_), "SPMM_TC");
+        cute_spmm_plan_info(plan_, &info);
+        numRowPanelsSplit = info.numChunks;
+        format_ = hrpb.device;
+    }
 };
+
+// inc.h:71-83
+inline void spmm_coo(unsigned int *rows, unsigned int *cols, float *vals, float *B, float *C, uint32_t M, uint32_t K,
+                     uint32_t N, unsigned int NNZ)
+{
+    cute::check(cute_spmm_coo(rows, cols, vals, B, C, M, K, N, NNZ), "spmm_coo");
+}
 
 // inc.h:84-109
 inline float check_gemm_correctness_coo(float *C, float *C_HOST, uint32_t M, uint32_t N)

@@ -43,6 +43,29 @@ int main(int argc, char **argv)
             for (unsigned int i = 0; i < hrpb.numNNZ && !bad; ++i) bad += back.cols[i] != hrpb.cols[i] || back.vals[i] != hrpb.vals[i];
             std::printf("cache=%zu\n", bad);
         }
+        {   // the registry behind the reference-shaped SPMM_TC constructor, and spmm_coo (inc.h:71-83)
+            const bool found = HRPB::find(hrpb.blockedRowPtr) == &hrpb && HRPB::find(reader.rowPtr) == nullptr;
+            bool gone;
+            unsigned int *stale;
+            {
+                HRPB second(reader.M, reader.K, reader.rowPtr, reader.cols, reader.vals, /*upload=*/false);
+                stale = second.blockedRowPtr;
+                gone = HRPB::find(stale) == &second;
+            }
+            gone = gone && HRPB::find(stale) == nullptr;
+            bool refused = false;
+            try {
+                SPMM_TC plan(reader.M, reader.K, 32, reader.rowPtr);      // not a format's blockedRowPtr
+            } catch (const cute::Error &e) {
+                refused = e.status == CUTE_ERR_ARG;
+            }
+            unsigned int rows[3] = {1, 0, 1}, cols[3] = {0, 1, 0};
+            float vals[3] = {2.0f, 3.0f, 4.0f}, B[4] = {1.0f, 10.0f, 100.0f, 1000.0f}, C[4];
+            spmm_coo(rows, cols, vals, B, C, 2, 2, 2, 3);
+            const bool coo = C[0] == 300.0f && C[1] == 3000.0f && C[2] == 6.0f && C[3] == 60.0f;
+            std::printf("registry=%d%d%d coo=%d fit=%d%d\n", int(found), int(gone), int(refused), int(coo),
+                        cute_offsets_fit(4096, 4096, 16, 0, (1u << 20) * 16ull), cute_offsets_fit(4096, 4096, 16, 0, (1u << 20) * 16ull - 16));
+        }
         try {
             MTX_READER missing("/nonexistent/file.mtx");
             return 3;

@@ -26,6 +26,7 @@ def test_reference_style_host_program(cs, orc, tmp_path):
     assert (int(got["panels"]), int(got["blocks"]), int(got["words"])) == (h["numRowPanels"], h["numBlocks"], h["numWords"])
     assert got["bcsr"] == "8750" and got["tiles"] == "4325" and got["heavy"] == "1875/33800" and got["light"] == "2450/6200"
     assert got["densediff"] == "0" and got["grown"] == "2,1" and got["cache"] == "0"
+    assert got["registry"] == "111" and got["coo"] == "1" and got["fit"] == "01"
     dy, dx, _, r, c, v = orc.coo_read(mtx)
     rp2, cl2, _ = orc.coo_to_csr(dy, r, c, v)
     want = orc.get_stats(dy, dx, rp2, cl2, 16)
