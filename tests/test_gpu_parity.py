@@ -138,6 +138,45 @@ def test_reference_regime_metric(cs, orc, torch_cuda):
             assert cs.check_gemm_correctness_coo(ref, out) <= 1e-5, (N, name)
 
 
+@pytest.mark.parametrize("cfg,scale", [(1, 1.0), (2, 1.0), (3, 1.0), (4, 1.0), (5, 1 / 8.0)])
+def test_literal_tolerance_on_every_config_pattern(cs, orc, torch_cuda, cfg, scale):
+    """The reference's metric (inc.h:84-109) at its literal fp32 bar, 1e-5, on the sparsity pattern of every
+    benchmark configuration in the regime the reference evaluates it in: values |a| (no cancellation) and
+    B uniform in [0,1) (run.cu:24-27).  Every kernel path; the backward error is recorded beside it."""
+    A = cs.gen_config(cfg, scale)
+    vals = np.abs(A.vals)
+    N = cs.CONFIGS[cfg]["N"]
+    B = cs.gen_dense(cs.SEED_BASE + 300 + cfg, A.K, N, 0)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, vals, B)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, vals)
+    worst = {}
+    big = A.nnz > 4_000_000
+    for name, kw in _paths(cs):
+        if big and name in ("brick_rolling_g2", "brick_pipelined_g2", "mfma_default"):
+            continue                                   # the largest pattern: one variant per kernel family is enough
+        out, _ = _run(cs, torch_cuda, h, B, **kw)
+        worst[name] = cs.check_gemm_correctness_coo(ref, out)
+        assert worst[name] <= 1e-5, (cfg, name, worst[name])
+    out, _ = _run(cs, torch_cuda, h, B)
+    print("cfg%d literal metric max %.3g, backward error %.3g" %
+          (cfg, max(worst.values()), cs.backward_error(A.rowPtr, A.cols, vals, B, ref, out)))
+
+
+@pytest.mark.parametrize("cfg,scale", [(1, 1.0), (2, 1 / 4.0), (3, 1 / 4.0), (4, 1 / 4.0), (5, 1 / 32.0)])
+@pytest.mark.parametrize("N", [32, 128, 512])
+def test_literal_tolerance_at_the_reference_widths(cs, orc, torch_cuda, cfg, scale, N):
+    """The three feature widths of the reference's driver (run.cu:16) on each (scaled) configuration pattern."""
+    A = cs.gen_config(cfg, scale)
+    vals = np.abs(A.vals)
+    B = cs.gen_dense(cs.SEED_BASE + 400 + cfg + N, A.K, N, 0)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, vals, B)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, vals)
+    for name, kw in _paths(cs):
+        out, _ = _run(cs, torch_cuda, h, B, **kw)
+        m = cs.check_gemm_correctness_coo(ref, out)
+        assert m <= 1e-5, (cfg, N, name, m)
+
+
 def test_edge_shapes(cs, orc, torch_cuda):
     from test_oracle_pins import _edge_cases
     rng = np.random.default_rng(0)
