@@ -26,7 +26,7 @@ ABI_SYMBOLS = [
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
-    "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run",
+    "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run", "cute_spmm_run_static",
     "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
     "cute_device_info",
     "cute_coo_read", "cute_coo_save_mtx", "cute_coo_release", "cute_coo_to_csr", "cute_csr_i32_release",
@@ -46,7 +46,7 @@ class CuteError(RuntimeError):
     def __init__(self, status, where):
         self.status = status
         msg = "%s: %s (%d)" % (where, _status_string(status), status)
-        if status == -7 or status == -8:
+        if status in (-7, -8, -10):
             msg += " -- " + _last_hip_error()
         super().__init__(msg)
 
@@ -85,7 +85,7 @@ class cute_plan_info(C.Structure):
                 ("numAtomicChunks", C.c_uint32), ("numBrickPanels", C.c_uint32), ("numRowPanelsSparse", C.c_uint32),
                 ("numEmptyPanels", C.c_uint32), ("slots", C.c_uint32), ("precision", C.c_uint32),
                 ("path", C.c_uint32), ("mfmaShape", C.c_uint32), ("pipeline", C.c_uint32),
-                ("fusedLaunch", C.c_uint32), ("dealtChunks", C.c_uint32), ("reserved", C.c_uint32 * 1)]
+                ("fusedLaunch", C.c_uint32), ("dealtChunks", C.c_uint32), ("partialTileKiB", C.c_uint32)]
 
 
 i32p = C.POINTER(C.c_int32)
@@ -121,6 +121,7 @@ class cute_block_class(C.Structure):
                 ("overloads", C.c_int32), ("kind", C.c_int32)]
 
 
+STATIC_SCRATCH_BYTES = 32 << 20      # CUTE_STATIC_SCRATCH_BYTES
 PATH_AUTO, PATH_BRICK, PATH_ROWS = 0, 1, 2
 PREC_FP32, PREC_BF16X3 = 0, 1
 
@@ -185,6 +186,7 @@ def load_library():
     lib.cute_spmm_plan_info.argtypes = [C.c_void_p, C.POINTER(cute_plan_info)]
     lib.cute_spmm_plan_free.argtypes = [C.c_void_p]
     lib.cute_spmm_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.cute_spmm_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.cute_csr_spmm_dev.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_uint32, C.c_uint32, C.c_void_p]
     lib.cute_gpu_csr_spmm.restype = C.c_float
@@ -557,6 +559,13 @@ class SPMM_TC:
         self._check_shapes(MatB, MatC)
         _check(load_library().cute_spmm_run(self._plan, _dev_ptr(MatB), _dev_ptr(MatC), _stream_ptr(stream)),
                "cute_spmm_run")
+        return MatC
+
+    def run_static(self, MatB, MatC, stream=None):
+        """``run`` without any allocation behind it: partial tiles go to the library's static device array."""
+        self._check_shapes(MatB, MatC)
+        _check(load_library().cute_spmm_run_static(self._plan, _dev_ptr(MatB), _dev_ptr(MatC), _stream_ptr(stream)),
+               "cute_spmm_run_static")
         return MatC
 
     def time(self, MatB, MatC, warmup=3, iters=20, stream=None):

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <mutex>
 #include <string>
 
 #include "common.hpp"
@@ -60,6 +61,31 @@ const DeviceContext &context()
     return ctx;
 }
 
+// Scratch for cute_spmm_run_static: the partial tiles of cut panels, for callers that cannot allocate.
+// One copy per GPU, part of the loaded code object, held until the process ends.  In host code the name
+// of the array is only a handle for hipGetSymbolAddress -- never a device address.
+static __device__ __align__(256) unsigned char scratch[CUTE_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void **out)
+{
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return CUTE_ERR_ARG;
+    std::lock_guard<std::mutex> g(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return CUTE_OK;
+}
+
 template <class T>
 int upload(T **dst, const T *src, uint64_t count)
 {
@@ -106,6 +132,7 @@ struct cute_spmm_plan {
     uint32_t numFixups = 0;
     uint32_t unitRows = CUTE_TM;        // rows of one panel / strip / piece
     float *dPartials = nullptr;         // pieces x unitRows rows of N floats; owned by the plan, so a plan runs on one stream at a time
+    uint64_t partialBytes = 0;
     uint32_t *dRowList = nullptr;
     uint32_t numRows = 0;
     cute_dev::XcdRanges rowRanges{};   // row-kernel blocks of each XCD, balanced by nonzeros
@@ -569,9 +596,16 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (rc == CUTE_OK && n_pieces) {
         // (the fast kernels address the partial tiles like C, with 32-bit byte offsets: checked where the chunks were made)
         const uint64_t bytes = uint64_t(n_pieces) * p->unitRows * N * sizeof(float);
+        p->partialBytes = bytes;
         if (hipMalloc(reinterpret_cast<void **>(&p->dPartials), bytes) != hipSuccess) rc = CUTE_ERR_NOMEM;
     }
     if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
+    if (rc == CUTE_OK) {
+        // cute_spmm_run_static's scratch: its address on this device is looked up here, at set-up, so that the
+        // run call itself is nothing but kernel launches
+        void *unused = nullptr;
+        rc = static_scratch(&unused);
+    }
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
     p->numFixups = uint32_t(fixups.size());
     p->numRows = uint32_t(row_list.size());
@@ -592,6 +626,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // kernel in the shapes the planner itself picks for N (forced column groups fall back to two launches)
     const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
     const bool brick_default_shape = ng_for_mixed || p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
+    p->info.partialTileKiB = uint32_t((p->partialBytes + 1023u) / 1024u);
     p->info.fusedLaunch = (rows_fusable && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
@@ -602,24 +637,24 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
 namespace {
 
 template <int VEC, int NG, bool FULL>
-void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, float *partials, hipStream_t s)
 {
     const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
     if (p->pipeline == 1)
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, NG, FULL>), grid, block, 0, s, p->dChunks,
-                           p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, p->dPartials, p->info.N);
+                           p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, partials, p->info.N);
     else
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32<VEC, NG, FULL>), grid, block, 0, s, p->dChunks, p->info.numChunks,
-                           per_xcd, p->d->dHdr, p->d->dVals, dB, dC, p->dPartials, p->info.N);
+                           per_xcd, p->d->dHdr, p->d->dVals, dB, dC, partials, p->info.N);
 }
 
 template <int VEC, int NG>
-void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, float *partials, hipStream_t s)
 {
-    if (p->info.N % p->info.slabWidth == 0) launch_brick_full<VEC, NG, true>(p, dB, dC, s);
-    else launch_brick_full<VEC, NG, false>(p, dB, dC, s);
+    if (p->info.N % p->info.slabWidth == 0) launch_brick_full<VEC, NG, true>(p, dB, dC, partials, s);
+    else launch_brick_full<VEC, NG, false>(p, dB, dC, partials, s);
 }
 
 template <int VEC, bool BATCHED>
@@ -743,7 +778,7 @@ namespace {
 // Brick chunks and sparse rows in one launch.  (VEC, NG, lanes per row) follow from N the way the planner
 // picks them; returns false for a combination that is not instantiated (the caller then launches twice).
 template <int VEC, int NG, int LOG_L>
-void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s, const dim3 &grid,
+void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, float *partials, hipStream_t s, const dim3 &grid,
                           uint32_t per_xcd)
 {
     const uint32_t N = p->info.N;
@@ -753,26 +788,26 @@ void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, h
     hipLaunchKernelGGL((cute_dev::hrpb_brick_rows_f32<VEC, NG, F, LOG_L>), flat, block, 0, s, grid.x, uint32_t(brick_blocks),  \
                        p->dChunks, p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), p->dRowList, \
                        p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals,                    \
-                       dB, dC, p->dPartials, N)
+                       dB, dC, partials, N)
     if (N % (16u * VEC * NG) == 0) CUTE_BRICK_ROWS(true);
     else CUTE_BRICK_ROWS(false);
 #undef CUTE_BRICK_ROWS
 }
 
-bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, hipStream_t s)
+bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, float *partials, hipStream_t s)
 {
     const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs);
     if (uint64_t(grid.x) * grid.y + uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd >= 0x7fffffffull) return false;
     const int v = p->vec, g = p->ng, l = p->rows_logl;
-    if (v == 1 && g == 1 && l == 2) launch_brick_rows_as<1, 1, 2>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 2 && g == 1 && l == 3) launch_brick_rows_as<2, 1, 3>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 4 && g == 1 && l == 4) launch_brick_rows_as<4, 1, 4>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 4 && g == 1 && l == 5) launch_brick_rows_as<4, 1, 5>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 4 && g == 1 && l == 6) launch_brick_rows_as<4, 1, 6>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 4 && g == 2 && l == 5) launch_brick_rows_as<4, 2, 5>(p, dB, dC, s, grid, per_xcd);
-    else if (v == 4 && g == 2 && l == 6) launch_brick_rows_as<4, 2, 6>(p, dB, dC, s, grid, per_xcd);
+    if (v == 1 && g == 1 && l == 2) launch_brick_rows_as<1, 1, 2>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 2 && g == 1 && l == 3) launch_brick_rows_as<2, 1, 3>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 4) launch_brick_rows_as<4, 1, 4>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 5) launch_brick_rows_as<4, 1, 5>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 4 && g == 1 && l == 6) launch_brick_rows_as<4, 1, 6>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 4 && g == 2 && l == 5) launch_brick_rows_as<4, 2, 5>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 4 && g == 2 && l == 6) launch_brick_rows_as<4, 2, 6>(p, dB, dC, partials, s, grid, per_xcd);
     else return false;
     return true;
 }
@@ -780,9 +815,11 @@ bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, hipS
 
 extern "C" {
 
-// Replaces SPMM_TC::run (spmm.cu:823-839): picks the kernel instantiation from N and
-// launches asynchronously on `stream`.
-int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
+}  // extern "C"
+
+namespace {
+// The launches of one product; `partials` is where the pieces of cut panels store their tiles.
+int run_with(const cute_spmm_plan *p, const float *dB, float *dC, void *stream, float *partials)
 {
     if (!p || !dB || !dC) return CUTE_ERR_ARG;
     if ((reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC)) & 15u) return CUTE_ERR_ARG;
@@ -802,7 +839,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
                        grid.x, uint32_t(quad_blocks), p->dHeads, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,   \
                        uint32_t(p->d->numQuadVals),                                                                  \
                        p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC,    \
-                       p->dPartials, N)
+                       partials, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
         case 2: CUTE_FUSED_LAUNCH(F, S, 2); break;                              \
@@ -821,7 +858,7 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
         } else {
 #define CUTE_QUAD_LAUNCH(F, S)                                                                                          \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_f32<F, S>), grid, block, 0, s, p->dHeads, p->info.numChunks, per_xcd,         \
-                       p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, p->dPartials, N)
+                       p->d->dQRecs, p->d->dQVals, uint32_t(p->d->numQuadVals), dB, dC, partials, N)
         if (full && strips) CUTE_QUAD_LAUNCH(true, true);
         else if (full) CUTE_QUAD_LAUNCH(true, false);
         else if (strips) CUTE_QUAD_LAUNCH(false, true);
@@ -829,11 +866,11 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
 #undef CUTE_QUAD_LAUNCH
         }
     } else if (p->info.numChunks) {
-        if (p->info.fusedLaunch && launch_brick_rows(p, dB, dC, s)) rows_launched = true;
-        else if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, s);
-        else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, s);
-        else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, s);
-        else launch_brick<1, 1>(p, dB, dC, s);
+        if (p->info.fusedLaunch && launch_brick_rows(p, dB, dC, partials, s)) rows_launched = true;
+        else if (p->vec == 4 && p->ng == 2) launch_brick<4, 2>(p, dB, dC, partials, s);
+        else if (p->vec == 4) launch_brick<4, 1>(p, dB, dC, partials, s);
+        else if (p->vec == 2) launch_brick<2, 1>(p, dB, dC, partials, s);
+        else launch_brick<1, 1>(p, dB, dC, partials, s);
     }
     if (p->numRows && !rows_launched) {
         // every row: no list needed, which takes one dependent load out of each row's chain
@@ -845,8 +882,35 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
     if (p->numFixups)
         hipLaunchKernelGGL(cute_dev::reduce_partials, dim3(p->numFixups, (p->unitRows * N + 63u) / 64u),
                            dim3(cute_dev::kWaveSize * cute_dev::kReduceWaves), 0, s, p->dFixups, p->numFixups, p->unitRows,
-                           p->dPartials, dC, N);
+                           partials, dC, N);
     return check_launch("spmm launch");
+}
+}  // namespace
+
+extern "C" {
+
+// Replaces SPMM_TC::run (spmm.cu:823-839): picks the kernel instantiation from N and
+// launches asynchronously on `stream`.
+int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
+{
+    if (!p) return CUTE_ERR_ARG;
+    return run_with(p, dB, dC, stream, p->dPartials);
+}
+
+// The same launches with the partial tiles in the library's static device array instead of the plan's
+// buffer: no allocation, no copy, no memset, no synchronisation -- kernel launches only.
+int cute_spmm_run_static(cute_spmm_plan *p, const float *dB, float *dC, void *stream)
+{
+    if (!p) return CUTE_ERR_ARG;
+    if (p->partialBytes > uint64_t(CUTE_STATIC_SCRATCH_BYTES)) {
+        g_hip_error = "plan needs " + std::to_string(p->partialBytes) + " bytes of partial tiles, the static scratch holds " +
+                      std::to_string(uint64_t(CUTE_STATIC_SCRATCH_BYTES));
+        return CUTE_ERR_SCRATCH;
+    }
+    void *ptr = nullptr;
+    const int rc = static_scratch(&ptr);      // a table look-up: the address was fetched when the plan was made
+    if (rc != CUTE_OK) return rc;
+    return run_with(p, dB, dC, stream, static_cast<float *>(ptr));
 }
 
 int cute_csr_spmm_dev(int alg, const uint32_t *dRowPtr, const uint32_t *dCols, const float *dVals, const float *dB,

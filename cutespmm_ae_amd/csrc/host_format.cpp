@@ -25,6 +25,7 @@ const char *cute_status_string(int s)
         case CUTE_ERR_HIP: return "HIP runtime error";
         case CUTE_ERR_NO_DEVICE: return "no gfx950 device";
         case CUTE_ERR_FORMAT: return "format stream failed validation";
+        case CUTE_ERR_SCRATCH: return "the plan's partial tiles do not fit the static scratch buffer";
         default: return "unknown status";
     }
 }

@@ -41,7 +41,8 @@ typedef enum cute_status {
     CUTE_ERR_NOMEM = -6,
     CUTE_ERR_HIP = -7,         /* a HIP runtime call failed; see cute_last_hip_error()    */
     CUTE_ERR_NO_DEVICE = -8,   /* no gfx950 device visible                                */
-    CUTE_ERR_FORMAT = -9       /* a format stream failed validation                       */
+    CUTE_ERR_FORMAT = -9,      /* a format stream failed validation                       */
+    CUTE_ERR_SCRATCH = -10     /* cute_spmm_run_static: the plan needs more scratch than the static buffer holds */
 } cute_status;
 
 const char *cute_status_string(int status);
@@ -370,7 +371,7 @@ typedef struct cute_plan_info {
     uint32_t pipeline;         /* brick kernel variant in use: 1 rolling, 2 pipelined     */
     uint32_t fusedLaunch;      /* 1: MFMA chunks and sparse rows go out as one launch     */
     uint32_t dealtChunks;      /* 1: the MFMA work items were dealt to the SIMDs by length (cute_tunables.chunk_order) */
-    uint32_t reserved[1];
+    uint32_t partialTileKiB;   /* KiB of partial tiles the pieces of cut panels store per launch (0: no panel is cut) */
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;
@@ -385,6 +386,19 @@ void cute_spmm_plan_free(cute_spmm_plan *p);
  * keeps their partial tiles in a buffer of its own: launches of ONE plan must not overlap in
  * time (same stream, or ordered by events); different plans are independent. */
 int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
+
+/* cute_spmm_run for callers that cannot allocate device memory (code under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels, same
+ * arguments, same bits in C; the partial tiles of cut panels go to a static device array of
+ * CUTE_STATIC_SCRATCH_BYTES that the library's code object carries (one copy per GPU, held until the
+ * process ends) instead of the plan's own buffer.  The call launches kernels and does nothing else: no
+ * hipMalloc/hipFree, no copy, no memset, no synchronisation.  A plan whose partial tiles
+ * (cute_plan_info.partialTileKiB) exceed the array gives CUTE_ERR_SCRATCH, and cute_last_hip_error()
+ * then names both sizes.  Every call on a GPU shares that GPU's array: calls that may overlap in time
+ * on one GPU -- of any plans -- race; order them (one stream, or events).  Nothing in the array has to
+ * start at zero: every piece overwrites its whole tile before the adding kernel reads it. */
+#define CUTE_STATIC_SCRATCH_BYTES (32u << 20)
+int cute_spmm_run_static(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
 
 /* ------------------------------------------------------------------------------------
  * device: plain CSR SpMM kernels -- the fp32 CSR comparison path.  Replaces
