@@ -500,15 +500,23 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
             // the mean only counts while it is short: a matrix whose few MFMA panels are all very long
             // (a handful of dense rows) must still be cut, or one wavefront walks a whole panel alone
             const uint32_t target = uint32_t(std::max<uint64_t>(std::max<uint64_t>(share, std::min<uint64_t>(mean, 16)), 8));
+            // A launch that keeps every wavefront slot busy runs at the rate the memory system gathers B rows, and a
+            // work item then advances about five times slower than one that runs alone (measured on the R-MAT
+            // benchmark matrix: 0.39 us per list group alone, 1.7 us per group and slot under load).  So an item up to
+            // six shares long still ends with the launch, and cutting it finer only adds partial tiles: such a launch
+            // cuts at six shares, into pieces of four.  A launch that does not fill the device is bound by its longest
+            // item instead and keeps the finer cut (twice the target, pieces of one target).
+            const uint32_t limit = uint32_t(std::max<uint64_t>(2u * uint64_t(target), 6u * share));
+            const uint32_t piece = limit > 2u * target ? uint32_t(4u * share) : target;
             for (uint32_t q = 0; q < num_units; ++q) {
                 const uint32_t s = unit[q], e = unit[q + 1];
                 if (s == e || to_rows[q / upp]) continue;
                 const uint32_t nblk = e - s;
-                if (nblk <= 2 * target) {
+                if (nblk <= limit) {
                     quads.insert(quads.end(), {s, e, q, 0u});
                     continue;
                 }
-                const uint32_t pieces = (nblk + target - 1) / target;
+                const uint32_t pieces = (nblk + piece - 1) / piece;
                 const uint32_t step = (nblk + pieces - 1) / pieces;
                 for (uint32_t cs = s; cs < e; cs += step) quads.insert(quads.end(), {cs, std::min(e, cs + step), q, 1u});
             }
@@ -574,8 +582,50 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         for (uint32_t k = 0; k < cute_dev::kNumXcd; ++k)
             p->rowBlocksPerXcd = std::max(p->rowBlocksPerXcd, p->rowRanges.first[k + 1] - p->rowRanges.first[k]);
     }
-    if (t.chunk_order > 2) { delete p; return CUTE_ERR_ARG; }
+    if (t.chunk_order > 3) { delete p; return CUTE_ERR_ARG; }
     p->info.dealtChunks = 0;
+    // A launch larger than the device starts its work-groups in list order as slots come free.  If its items differ
+    // widely in length (the longest at least four times the mean), the long ones go first, so that they run from the
+    // start and the short ones fill the gaps they leave; items are ordered by the power of two of their length only,
+    // so neighbours of similar length stay neighbours and keep sharing B rows in the L2.
+    bool longest_first = t.chunk_order == 3;
+    if (t.chunk_order == 0 && !chunks.empty()) {
+        const uint64_t resident = uint64_t(c.num_cus) * 4u * ((p->shape == 2 || p->ng == 1) ? 8u : 4u);
+        uint64_t total = 0;
+        uint32_t longest = 0;
+        for (const uint4 &ck : chunks) { total += ck.y - ck.x; longest = std::max(longest, ck.y - ck.x); }
+        longest_first = uint64_t(chunks.size()) * num_slabs > resident && uint64_t(longest) * chunks.size() >= 4u * total;
+    }
+    if (longest_first && !chunks.empty()) {
+        std::vector<uint4> sorted(chunks);
+        std::stable_sort(sorted.begin(), sorted.end(), [](const uint4 &a, const uint4 &b) {
+            return __builtin_clz((a.y - a.x) | 1u) < __builtin_clz((b.y - b.x) | 1u);
+        });
+        // work-group g runs on XCD g % 8 and takes the list positions the kernels' XCD mapping gives it: XCD x walks
+        // the groups [x * per_xcd, (x + 1) * per_xcd).  Deal the sorted groups round-robin into those ranges.
+        const uint32_t wpg = cute_dev::kWavesPerGroup;
+        const uint32_t groups = (uint32_t(sorted.size()) + wpg - 1) / wpg;
+        const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+        uint32_t fill[cute_dev::kNumXcd] = {}, cap[cute_dev::kNumXcd];
+        for (uint32_t x = 0; x < cute_dev::kNumXcd; ++x)
+            cap[x] = uint32_t(std::min<uint64_t>(per_xcd, groups > x * per_xcd ? groups - x * per_xcd : 0));
+        // the last group may be short: it must stay the last one of the list
+        const bool ragged = sorted.size() % wpg != 0;
+        uint32_t last_xcd = 0;
+        for (uint32_t x = 0; x < cute_dev::kNumXcd; ++x) if (cap[x]) last_xcd = x;
+        if (ragged) cap[last_xcd]--;
+        for (uint32_t k = 0; k < groups - (ragged ? 1u : 0u); ++k) {
+            uint32_t x = k % cute_dev::kNumXcd;
+            while (fill[x] == cap[x]) x = (x + 1) % cute_dev::kNumXcd;
+            const size_t dst = (size_t(x) * per_xcd + fill[x]++) * wpg;
+            for (uint32_t w = 0; w < wpg; ++w) chunks[dst + w] = sorted[size_t(k) * wpg + w];
+        }
+        if (ragged) {
+            const size_t dst = (size_t(last_xcd) * per_xcd + cap[last_xcd]) * wpg, src = size_t(groups - 1) * wpg;
+            for (size_t w = 0; src + w < sorted.size(); ++w) chunks[dst + w] = sorted[src + w];
+        }
+        p->info.dealtChunks = 2;
+    } else
     if (t.chunk_order != 1 && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
         p->info.dealtChunks = deal_chunks(chunks, num_slabs, uint32_t(c.num_cus) / cute_dev::kNumXcd,
                                           p->shape == 2 || p->ng == 1 ? 8u : 4u, t.chunk_order == 2) ? 1u : 0u;

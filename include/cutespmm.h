@@ -353,8 +353,9 @@ typedef struct cute_tunables {
     uint32_t pipeline;         /* brick kernel variant: 1 rolling, 2 pipelined; 0: default (rolling)             */
     uint32_t mfma_shape;       /* MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists; 0: chosen per matrix (list slots per brick) */
     uint32_t max_row_nnz;      /* AUTO: panels holding a row longer than this stay on the brick kernel; 0: default  */
-    uint32_t chunk_order;      /* MFMA work items: 0 dealt to the SIMDs longest first where the whole launch is resident and that
-                                  shortens the fullest SIMD; 1 always in panel order; 2 always dealt */
+    uint32_t chunk_order;      /* MFMA work items: 0 library's choice (a launch that is resident at once: dealt to the SIMDs longest
+                                  first where that shortens the fullest SIMD; a larger launch whose longest item is four times the
+                                  mean: long items first); 1 always in panel order; 2 always dealt; 3 always long items first */
     uint32_t reserved[2];
 } cute_tunables;
 
@@ -370,7 +371,7 @@ typedef struct cute_plan_info {
     uint32_t mfmaShape;        /* MFMA kernel in use: 1 16x16x4 bricks, 2 4x4x1 quad lists */
     uint32_t pipeline;         /* brick kernel variant in use: 1 rolling, 2 pipelined     */
     uint32_t fusedLaunch;      /* 1: MFMA chunks and sparse rows go out as one launch     */
-    uint32_t dealtChunks;      /* 1: the MFMA work items were dealt to the SIMDs by length (cute_tunables.chunk_order) */
+    uint32_t dealtChunks;      /* 1: the MFMA work items were dealt to the SIMDs by length, 2: listed long items first, 0: panel order (cute_tunables.chunk_order) */
     uint32_t partialTileKiB;   /* KiB of partial tiles the pieces of cut panels store per launch (0: no panel is cut) */
 } cute_plan_info;
 

@@ -239,13 +239,13 @@ def test_work_items_dealt_by_length(cs, orc, torch_cuda):
         ref = orc.spmm_csr(rp, cl, vl, B)
         for kw in (dict(path=cs.PATH_BRICK, mfma_shape=1), dict(path=cs.PATH_BRICK, mfma_shape=2), dict()):
             outs = {}
-            for order in (1, 0, 2):
+            for order in (1, 0, 2, 3):
                 outs[order], plan = _run(cs, torch_cuda, h, B, chunk_order=order, **kw)
-                assert plan.info["dealtChunks"] == (0 if order == 1 else 1 if order == 2 else plan.info["dealtChunks"])
+                assert plan.info["dealtChunks"] == (0 if order == 1 else 1 if order == 2 else 2 if order == 3 else plan.info["dealtChunks"])
                 if order == 1 and "path" in kw:
                     assert plan.info["numAtomicChunks"] > 0
             assert cs.backward_error(rp, cl, vl, B, ref, outs[1]) <= BERR, (N, kw)
-            assert (outs[0] == outs[1]).all() and (outs[2] == outs[1]).all(), (N, kw)
+            assert (outs[0] == outs[1]).all() and (outs[2] == outs[1]).all() and (outs[3] == outs[1]).all(), (N, kw)
     # several work items per SIMD, of very different lengths, all on the device at once: the planner deals them by itself
     M3, K3 = 32768, 2048
     lengths = rng.integers(1, 24, M3 // 16)
@@ -259,13 +259,27 @@ def test_work_items_dealt_by_length(cs, orc, torch_cuda):
         assert cs.backward_error(rp3, cl3, vl3, B3, ref3, out) <= BERR
         same, plan = _run(cs, torch_cuda, h3, B3, path=cs.PATH_BRICK, mfma_shape=shape, chunk_order=1)
         assert plan.info["dealtChunks"] == 0 and (same == out).all()
+    # a launch larger than the device with a heavy tail of long panels: the planner lists the long items first by
+    # itself, and cuts at a multiple of the per-slot share; same bits as panel order
+    M4, K4 = 65536, 8192
+    hub = set(int(x) for x in rng.choice(M4, 40, replace=False))
+    rp4, cl4, vl4 = random_csr(rng, M4, K4, row_nnz=lambda r: 3000 if r in hub else 3)
+    h4 = cs.HRPB(M4, K4, rp4, cl4, vl4)
+    B4 = rng.standard_normal((K4, 192)).astype(np.float32)
+    ref4 = orc.spmm_csr(rp4, cl4, vl4, B4)
+    for shape in (1, 2):
+        out, plan = _run(cs, torch_cuda, h4, B4, path=cs.PATH_BRICK, mfma_shape=shape)
+        assert plan.info["dealtChunks"] == 2 and plan.info["numAtomicChunks"] > 0, plan.info
+        assert cs.backward_error(rp4, cl4, vl4, B4, ref4, out) <= BERR
+        same, plan = _run(cs, torch_cuda, h4, B4, path=cs.PATH_BRICK, mfma_shape=shape, chunk_order=1)
+        assert plan.info["dealtChunks"] == 0 and (same == out).all()
     # equal panels stay in panel order
     rp2, cl2, vl2 = random_csr(rng, 1024, 1024, row_nnz=lambda r: 8)
     h2 = cs.HRPB(1024, 1024, rp2, cl2, vl2)
     _, plan = _run(cs, torch_cuda, h2, rng.standard_normal((1024, 64)).astype(np.float32), path=cs.PATH_BRICK, mfma_shape=1)
     assert plan.info["dealtChunks"] == 0
     with pytest.raises(cs.CuteError):
-        cs.SPMM_TC(h2, 64, chunk_order=3)
+        cs.SPMM_TC(h2, 64, chunk_order=4)
 
 
 def test_csr_comparison_kernels(cs, orc, torch_cuda):
@@ -330,7 +344,7 @@ def test_plan_rejects_bad_arguments(cs, torch_cuda):
     long_panel = cs.HRPB(64, 4096, rp, cl, vl)
     assert cs.SPMM_TC(long_panel, 128, path=cs.PATH_BRICK).info["numAtomicChunks"] > 0
     with pytest.raises(cs.CuteError) as e:
-        cs.SPMM_TC(long_panel, 300000, path=cs.PATH_BRICK)
+        cs.SPMM_TC(long_panel, 300000, path=cs.PATH_BRICK, max_chunk_blocks=4)
     assert e.value.status == -2
     assert cs.SPMM_TC(h, 300000, path=cs.PATH_BRICK).info["numAtomicChunks"] == 0
 
