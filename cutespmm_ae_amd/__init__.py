@@ -549,6 +549,7 @@ class SPMM_TC:
         self.numRowPanelsSplit = info.numChunks
         self.kernel_name = (("hrpb_quad_rows_f32" if info.fusedLaunch else "hrpb_quad_f32") if info.mfmaShape == 2 else
                             "hrpb_brick_rows_f32" if info.fusedLaunch else
+                            "hrpb_brick_bf16x3" if info.precision == PREC_BF16X3 else
                             "hrpb_brick_f32_rolling" if info.pipeline == 1 else "hrpb_brick_f32")
 
     def _check_shapes(self, MatB, MatC):

@@ -123,6 +123,7 @@ struct cute_spmm_plan {
     int vec = 4, ng = 1;                // brick kernel shape
     int pipeline = 1;                   // 1: rolling variant, 2: pipelined variant
     int shape = 2;                      // MFMA kernel: 1 16x16x4 bricks, 2 4x4x1 quad lists
+    bool bf16x3 = false;                // brick kernel on the bf16 matrix pipeline (three products of bf16 hi/lo parts)
     int rows_vec = 4, rows_logl = 6;    // row kernel shape
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
@@ -380,7 +381,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     cute_tunables t{};
     if (tn) t = *tn;
     if (t.path < CUTE_PATH_AUTO || t.path > CUTE_PATH_ROWS) return CUTE_ERR_ARG;
-    if (t.precision != CUTE_PREC_FP32) return CUTE_ERR_ARG;   // the bf16x3 kernel is not built yet
+    if (t.precision != CUTE_PREC_FP32 && t.precision != CUTE_PREC_BF16X3) return CUTE_ERR_ARG;
     const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : 1.25f;
     const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : 48;   // measured: longer rows serialise a lane group
     // An MFMA work item always spans 64 output columns; when N is narrower the row kernel wastes
@@ -445,6 +446,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (p->pipeline == 1 && !offsets_fit) p->pipeline = 2;
     if (t.mfma_shape > 2) { delete p; return CUTE_ERR_ARG; }
     if (t.mfma_shape) p->shape = int(t.mfma_shape);
+    else if (t.precision == CUTE_PREC_BF16X3) p->shape = 1;      // the reduced-precision kernel works on the brick tiles
     else {
         // A 16x4 brick costs the same matrix time however few nonzeros it holds; the quad lists
         // only pay for occupied (4-row group, column) pairs but fetch a B row once per row group
@@ -460,6 +462,8 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         p->shape = slots < 8u * bricks ? 2 : 1;
     }
     if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
+    // bf16x3 exists for the rolling brick kernel with four columns per lane; any other shape computes in fp32
+    p->bf16x3 = t.precision == CUTE_PREC_BF16X3 && p->shape == 1 && p->pipeline == 1 && p->vec == 4;
     // The chunk list depends on the MFMA kernel (its work units are blocks or list groups).  It is built,
     // and if the partial tiles of the cut panels then turn out to be more rows than the fast kernels'
     // 24-bit row operand can address, built once more for the pipelined brick kernel, whose stores use
@@ -552,6 +556,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         if (attempt || t.mfma_shape == 2 || t.pipeline == 1) { delete p; return CUTE_ERR_SHAPE; }   // the caller forced a fast kernel
         p->shape = 1;
         p->pipeline = 2;
+        p->bf16x3 = false;
     }
     std::vector<uint32_t> row_list;
     for (uint32_t q = 0; q < d->P; ++q)
@@ -668,7 +673,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     p->info.numRowPanelsSparse = n_rows;
     p->info.numEmptyPanels = n_empty;
     p->info.slots = slots;
-    p->info.precision = uint32_t(t.precision);
+    p->info.precision = p->bf16x3 ? uint32_t(CUTE_PREC_BF16X3) : uint32_t(CUTE_PREC_FP32);
     p->info.path = uint32_t(t.path);
     p->info.mfmaShape = uint32_t(p->shape);
     p->info.pipeline = uint32_t(p->pipeline);
@@ -677,7 +682,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
     const bool brick_default_shape = ng_for_mixed || p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
     p->info.partialTileKiB = uint32_t((p->partialBytes + 1023u) / 1024u);
-    p->info.fusedLaunch = (rows_fusable && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
+    p->info.fusedLaunch = (rows_fusable && !p->bf16x3 && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
 }
@@ -692,7 +697,11 @@ void launch_brick_full(const cute_spmm_plan *p, const float *dB, float *dC, floa
     const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
-    if (p->pipeline == 1)
+    if (p->bf16x3) {
+        if constexpr (VEC == 4)
+            hipLaunchKernelGGL((cute_dev::hrpb_brick_bf16x3<NG, FULL>), grid, block, 0, s, p->dChunks, p->info.numChunks, per_xcd,
+                               p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, partials, p->info.N);
+    } else if (p->pipeline == 1)
         hipLaunchKernelGGL((cute_dev::hrpb_brick_f32_rolling<VEC, NG, FULL>), grid, block, 0, s, p->dChunks,
                            p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), dB, dC, partials, p->info.N);
     else

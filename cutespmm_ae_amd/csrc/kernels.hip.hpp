@@ -419,6 +419,116 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
 }
 
 // ---------------------------------------------------------------------------------------
+// Reduced-precision brick kernel: the same tiles, loads and C layout as the rolling fp32 kernel, but the
+// products run on the bf16 matrix pipeline.  Every fp32 operand x is split in registers into two bf16
+// numbers, hi = bf16(x) and lo = bf16(x - hi) (round to nearest; x - hi is exact in fp32), and a block
+// contributes  A_hi.B_hi + A_lo.B_hi + A_hi.B_lo  -- three v_mfma_f32_16x16x16_bf16 with fp32
+// accumulation.  What is dropped (A_lo.B_lo and the rounding of the lo parts) is below 2^-16 of each
+// product.  One such instruction spans the 16 active columns of a whole block: k slot 4g+i of lane
+// group g is column g of brick i, which is exactly what lane group g of the fp32 kernel fetches for
+// brick i -- so the block header, the masked A fetch through the lane-order bitmaps and the B gathers are
+// those of the fp32 kernel unchanged, and only the arithmetic between the loads differs.  An fp32 block
+// costs 4 bricks x 32 cycles per 16 columns on the matrix pipeline, this one 3 x 16; the split costs
+// three vector instructions per B value, which (unlike next to fp32 MFMAs) overlap with bf16 MFMAs.
+// ---------------------------------------------------------------------------------------
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// hi and lo parts of four fp32 values as two packed bf16 quadruples
+__device__ __forceinline__ void split_bf16x4(float x0, float x1, float x2, float x3, s16x4 &hi, s16x4 &lo)
+{
+    const uint32_t h01 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){x0, x1}, bf16x2));
+    const uint32_t h23 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){x2, x3}, bf16x2));
+    const float r0 = x0 - __uint_as_float(h01 << 16), r1 = x1 - __uint_as_float(h01 & 0xffff0000u);
+    const float r2 = x2 - __uint_as_float(h23 << 16), r3 = x3 - __uint_as_float(h23 & 0xffff0000u);
+    const uint32_t l01 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){r0, r1}, bf16x2));
+    const uint32_t l23 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){r2, r3}, bf16x2));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    hi = __builtin_bit_cast(s16x4, (u32x2){h01, h23});
+    lo = __builtin_bit_cast(s16x4, (u32x2){l01, l23});
+}
+
+template <int NG>
+struct Bf16Operands {
+    s16x4 a_hi, a_lo;
+    s16x4 b_hi[NG][4], b_lo[NG][4];
+};
+
+template <int NG>
+__device__ __forceinline__ void split_block(Bf16Operands<NG> &o, const float (&a)[4], const f32x4 (&b)[4][NG])
+{
+    split_bf16x4(a[0], a[1], a[2], a[3], o.a_hi, o.a_lo);
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) split_bf16x4(b[0][ng][v], b[1][ng][v], b[2][ng][v], b[3][ng][v], o.b_hi[ng][v], o.b_lo[ng][v]);
+}
+
+template <int NG>
+__device__ __forceinline__ void mfma_block_bf16x3(const Bf16Operands<NG> &o, f32x4 (&acc)[NG][4])
+{
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(o.a_hi, o.b_hi[ng][v], acc[ng][v], 0, 0, 0);
+            acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(o.a_lo, o.b_hi[ng][v], acc[ng][v], 0, 0, 0);
+            acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(o.a_hi, o.b_lo[ng][v], acc[ng][v], 0, 0, 0);
+        }
+}
+
+template <int NG, bool FULL>
+__global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 6 : 4)) void hrpb_brick_bf16x3(
+    const uint4 *__restrict__ chunks, uint32_t num_chunks, uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr,
+    const float *__restrict__ vals, uint32_t zero_index, const float *__restrict__ B, float *__restrict__ C,
+    float *__restrict__ partials, uint32_t N)
+{
+    constexpr int VEC = 4;
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, blockIdx.x, blockIdx.y);
+    if (!it.valid) return;
+    const uint32_t end = it.end;
+    const uint32_t row_pitch = N * 4u, col_off = it.col0 * 4u;
+
+    f32x4 acc[NG][VEC];
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[ng][v] = f32x4(0.0f);
+
+    uint32_t blk = it.start;
+    if (blk < end) {
+        f32x4 b[4][NG];
+        float a[4];
+        LeanHeader h1;
+        {
+            const LeanHeader h0 = load_lean_header(hdr, blk, lane);
+            h1 = load_lean_header(hdr, min(blk + 1, end - 1), lane);
+            asm volatile("" ::"v"(h1.cols[0]), "v"(h1.cols[1]), "v"(h1.cols[2]), "v"(h1.cols[3]));   // as in the fp32 kernel
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+        }
+        Bf16Operands<NG> o;
+        // per block: split what has arrived, ask for the next block into the same registers, multiply
+        for (; blk + 1 < end; ++blk) {       // a/b hold block blk, h1 the header line of blk+1
+            const LeanHeader h2 = load_lean_header(hdr, min(blk + 2, end - 1), lane);
+            __builtin_amdgcn_sched_barrier(0);
+            split_block<NG>(o, a, b);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_block_bf16x3<NG>(o, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            h1 = h2;
+        }
+        split_block<NG>(o, a, b);
+        mfma_block_bf16x3<NG>(o, acc);
+    }
+    brick_store_lean<VEC, NG, FULL>(it, acc, C, partials, N, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Quad kernel: v_mfma_f32_4x4x1_16B_f32 over the quad lists (see cute_quad_lists).
 //
 // With cbsz = 4 the instruction takes the four A values of lanes 4p..4p+3 (abid = p), and

@@ -340,7 +340,10 @@ typedef enum cute_path {
 
 typedef enum cute_precision {
     CUTE_PREC_FP32 = 0,        /* fp32 MFMA (4x4x1 or 16x16x4), fp32 operands             */
-    CUTE_PREC_BF16X3 = 1       /* bf16 hi/lo split, three bf16 MFMA products              */
+    CUTE_PREC_BF16X3 = 1       /* brick kernel on the bf16 matrix pipeline: operands split into bf16 hi + lo in registers,
+                                  three products per block, fp32 accumulation; error below 2^-16 per product.  Used where it
+                                  exists (brick tiles, N a multiple of 4, 32-bit offsets), fp32 elsewhere: cute_plan_info.precision
+                                  says which.  Panels the planner sends to the row kernel are always fp32. */
 } cute_precision;
 
 typedef struct cute_tunables {

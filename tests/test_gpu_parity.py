@@ -177,6 +177,67 @@ def test_literal_tolerance_at_the_reference_widths(cs, orc, torch_cuda, cfg, sca
         assert m <= 1e-5, (cfg, N, name, m)
 
 
+BERR_BF16X3 = 5e-5      # three bf16 products per block: what is dropped is below 2^-16 of each product (measured 2e-5)
+
+
+def test_bf16x3_precision_path(cs, orc, torch_cuda):
+    """CUTE_PREC_BF16X3: the brick kernel on the bf16 matrix pipeline.  Backward error in the 2^-15 class on every
+    benchmark pattern, the reference's metric within its reduced-precision bar of 1e-3 (in fact 1e-4) in the
+    reference's regime, exact on small integers (their hi parts are exact and their lo parts zero), every
+    width, cut panels, and fp32 wherever the kernel does not exist."""
+    for cfg, scale in [(1, 1.0), (2, 1 / 16.0), (3, 1 / 8.0), (4, 1 / 32.0), (5, 1 / 128.0)]:
+        A = cs.gen_config(cfg, scale)
+        N = cs.CONFIGS[cfg]["N"]
+        B = cs.gen_dense(cs.SEED_BASE + 100 + cfg, A.K, N, 2)
+        ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+        h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+        for kw in (dict(path=cs.PATH_BRICK), dict(path=cs.PATH_BRICK, brick_groups=1), dict()):
+            out, plan = _run(cs, torch_cuda, h, B, precision=cs.PREC_BF16X3, **kw)
+            err = cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, out)
+            assert np.isfinite(out).all() and err <= BERR_BF16X3, (cfg, kw, err)
+            if "path" in kw and N > 32:                             # narrower products take two-column tiles, in fp32
+                assert plan.info["precision"] == cs.PREC_BF16X3 and plan.kernel_name == "hrpb_brick_bf16x3"
+                assert err > 1e-6                                   # it really is the reduced-precision kernel
+        # the reference's regime: A = |a|, B in [0,1)
+        vals = np.abs(A.vals)
+        B0 = cs.gen_dense(cs.SEED_BASE + 500 + cfg, A.K, N, 0)
+        ref0 = orc.spmm_csr(A.rowPtr, A.cols, vals, B0)
+        h0 = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, vals)
+        out, _ = _run(cs, torch_cuda, h0, B0, precision=cs.PREC_BF16X3, path=cs.PATH_BRICK)
+        assert cs.check_gemm_correctness_coo(ref0, out) <= 1e-4, cfg
+    rng = np.random.default_rng(23)
+    M, K = 160, 256
+    rp, cl, vl = random_csr(rng, M, K, density=0.08, values="ints")
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for N in (4, 20, 64, 100, 128, 192, 260, 512):
+        B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        out, plan = _run(cs, torch_cuda, h, B, precision=cs.PREC_BF16X3, path=cs.PATH_BRICK)
+        assert plan.info["precision"] == (cs.PREC_BF16X3 if N > 32 else cs.PREC_FP32) and (out == ref).all(), N
+    # widths the kernel does not exist for (N not a multiple of 4), the quad kernel, the pipelined brick kernel: fp32
+    B = rng.standard_normal((K, 30)).astype(np.float32)
+    out, plan = _run(cs, torch_cuda, h, B, precision=cs.PREC_BF16X3, path=cs.PATH_BRICK)
+    assert plan.info["precision"] == cs.PREC_FP32 and cs.backward_error(rp, cl, vl, B, orc.spmm_csr(rp, cl, vl, B), out) <= BERR
+    B = rng.standard_normal((K, 64)).astype(np.float32)
+    for kw in (dict(mfma_shape=2), dict(pipeline=2)):
+        out, plan = _run(cs, torch_cuda, h, B, precision=cs.PREC_BF16X3, path=cs.PATH_BRICK, **kw)
+        assert plan.info["precision"] == cs.PREC_FP32 and cs.backward_error(rp, cl, vl, B, orc.spmm_csr(rp, cl, vl, B), out) <= BERR
+    # cut panels: partial tiles added in fp32, in a fixed order
+    M, K, N = 512, 4096, 128
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1500 if r in (5, 300) else 4)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    outs = []
+    for kw in (dict(), dict(max_chunk_blocks=3), dict(max_chunk_blocks=3)):
+        out, plan = _run(cs, torch_cuda, h, B, precision=cs.PREC_BF16X3, path=cs.PATH_BRICK, **kw)
+        assert plan.info["numAtomicChunks"] > 0 and cs.backward_error(rp, cl, vl, B, ref, out) <= BERR_BF16X3
+        outs.append(out)
+    assert (outs[1] == outs[2]).all()
+    with pytest.raises(cs.CuteError):
+        cs.SPMM_TC(h, N, precision=2)
+
+
 def test_edge_shapes(cs, orc, torch_cuda):
     from test_oracle_pins import _edge_cases
     rng = np.random.default_rng(0)
