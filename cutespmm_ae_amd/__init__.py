@@ -22,7 +22,7 @@ ABI_SYMBOLS = [
     "cute_spmm_coo", "cute_offsets_fit",
     "cute_hrpb_build", "cute_hrpb_host_release",
     "cute_hrpb_retile", "cute_hrpb_untile", "cute_hrpb_tiled_release",
-    "cute_quad_build", "cute_quad_fill", "cute_quad_build_strips", "cute_quad_release", "cute_hrpb_save", "cute_hrpb_load",
+    "cute_quad_build", "cute_quad_fill", "cute_quad_build_strips", "cute_quad_release", "cute_quad_census", "cute_quad_pack", "cute_hrpb_save", "cute_hrpb_load",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
@@ -160,6 +160,8 @@ def load_library():
     lib.cute_hrpb_tiled_release.argtypes = [C.POINTER(cute_hrpb_tiled)]
     lib.cute_quad_build.argtypes = [C.c_uint32, C.c_uint32, u32p, u32p, f32p, C.POINTER(cute_quad_lists)]
     lib.cute_quad_build_strips.argtypes = lib.cute_quad_build.argtypes
+    lib.cute_quad_census.argtypes = [C.c_uint32, u32p, u32p, f32p, u32p, u32p]
+    lib.cute_quad_pack.argtypes = [C.c_uint32, u32p, u32p, f32p, C.c_uint32, u32p, u64p, u32p, f32p]
     lib.cute_hrpb_upload_layout.argtypes = [C.POINTER(cute_hrpb_host), C.c_int, C.POINTER(C.c_void_p)]
     lib.cute_quad_release.argtypes = [C.POINTER(cute_quad_lists)]
     lib.cute_quad_release.restype = None
@@ -521,6 +523,30 @@ def quad_lists(M, K, rowPtr, cols, vals, strips=False):
                vals=_view(q.vals, q.numGroups * 64, np.float32).reshape(-1, 64).copy())
     load_library().cute_quad_release(C.byref(q))
     return out
+
+
+def quad_pack(M, rowPtr, cols, vals, strips=False):
+    """The device form of the quad lists as ``cute_hrpb_upload`` builds it, straight from the CSR matrix:
+    dict(groupPtr[U+1], recs[G,20] = 16 columns + slot mask (2 words) + first value + 0, packed = stored values)."""
+    lib = load_library()
+    rowPtr, cols, vals = _as(rowPtr, np.uint32), _as(cols, np.uint32), _as(vals, np.float32)
+    S = (int(M) + 3) // 4
+    pairs, stored = np.zeros(S, np.uint32), np.zeros(S, np.uint32)
+    _check(lib.cute_quad_census(int(M), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p), _ptr(pairs, u32p),
+                                _ptr(stored, u32p)), "cute_quad_census")
+    if strips:
+        groups = (pairs.astype(np.int64) + 15) // 16
+        per_unit = stored.astype(np.int64)
+    else:
+        groups = (pairs.reshape(-1, 4).max(1).astype(np.int64) + 3) // 4
+        per_unit = stored.reshape(-1, 4).sum(1).astype(np.int64)
+    groupPtr = np.concatenate([[0], np.cumsum(groups)]).astype(np.uint32)
+    valBase = np.concatenate([[0], np.cumsum(per_unit)]).astype(np.uint64)
+    recs = np.zeros((int(groupPtr[-1]), 20), np.uint32)
+    packed = np.zeros(int(valBase[-1]), np.float32)
+    _check(lib.cute_quad_pack(int(M), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p), 4 if strips else 16,
+                              _ptr(groupPtr, u32p), _ptr(valBase, u64p), _ptr(recs, u32p), _ptr(packed, f32p)), "cute_quad_pack")
+    return dict(groupPtr=groupPtr, recs=recs, packed=packed, stripPairs=pairs, stripVals=stored)
 
 
 def _stream_ptr(stream):

@@ -14,6 +14,11 @@ namespace {
 
 thread_local std::string g_hip_error;
 
+// The planner's default thresholds (measured on the five benchmark matrices and on the reference's 43).
+constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
+constexpr uint32_t kMaxRowForRows = 48;     // ... unless it holds a row longer than this: one lane group would serialise it
+constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
+
 inline int hip_fail(hipError_t e, const char *what, int line)
 {
     g_hip_error = std::string(hipGetErrorString(e)) + " (" + what + ", device.hip:" + std::to_string(line) + ")";
@@ -100,8 +105,13 @@ int upload(T **dst, const T *src, uint64_t count)
 struct cute_hrpb_dev {
     uint32_t M = 0, K = 0, nnz = 0, P = 0, nb = 0;
     uint64_t numVals = 0, bytes = 0;
-    uint32_t *dHdr = nullptr;
-    float *dVals = nullptr;
+    // Of the two MFMA layouts only the one the planner's default rules would pick for this matrix is built by
+    // the upload (none if every panel would go to the row kernel); the other is built from the device copy of
+    // the CSR arrays the first time a plan asks for it.  `lock` guards those late builds.
+    std::mutex lock;
+    bool haveBricks = false, haveQuads = false;
+    uint32_t *dHdr = nullptr;           // brick tiles: one 128-byte header line per block
+    float *dVals = nullptr;             // brick tiles: values in lane order, then 64 zeros
     uint32_t *dRowPtr = nullptr, *dCols = nullptr;
     float *dCsrVals = nullptr;
     uint32_t *dQRecs = nullptr;         // quad lists: one record per group (16 columns, slot mask, first value)
@@ -109,7 +119,9 @@ struct cute_hrpb_dev {
     uint64_t numQuadVals = 0;
     uint64_t numGroups = 0;
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
-    std::vector<uint32_t> qgp;          // host copy of the quad lists' groupPtr
+    std::vector<uint32_t> qgp;          // the quad lists' groupPtr (known from the census, before the lists are built)
+    std::vector<uint64_t> qValBase;     // index of each list unit's first stored value
+    std::vector<uint32_t> qrecsHost;    // host copy of the group records (a plan copies its chunks' first records from it)
     uint32_t quadRows = CUTE_TM;        // rows per list unit: 16 (lockstep lists per panel) or 4 (strips)
     uint64_t quadPairs = 0;             // occupied (row group, column) pairs
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
@@ -240,22 +252,85 @@ uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d) { return d ? d->bytes : 0; 
 
 int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out) { return cute_hrpb_upload_layout(h, 0, out); }
 
+}  // extern "C"
+
+namespace {
+
+// Brick tiles of a canonical format onto the device.
+int build_bricks(cute_hrpb_dev *d, const cute_hrpb_host *h)
+{
+    cute_hrpb_tiled t;
+    int rc = cute_hrpb_retile(h, &t);
+    if (rc != CUTE_OK) return rc;
+    rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
+    if (rc == CUTE_OK) {
+        // one wavefront of zero padding behind the values: a lane without a nonzero reads its operand there
+        std::vector<float> padded(t.numVals + 64, 0.0f);
+        if (t.numVals) std::memcpy(padded.data(), t.vals, t.numVals * sizeof(float));
+        rc = upload(&d->dVals, padded.data(), padded.size());
+    }
+    if (rc == CUTE_OK) {
+        d->bytes += uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + (t.numVals + 64) * 4;
+        d->haveBricks = true;
+    }
+    cute_hrpb_tiled_release(&t);
+    return rc;
+}
+
+// Quad lists (in the layout chosen at upload) onto the device, straight from the CSR arrays.
+int build_quads(cute_hrpb_dev *d, const uint32_t *rowPtr, const uint32_t *cols, const float *vals)
+{
+    d->qrecsHost.assign(d->numGroups * CUTE_QUAD_RECORD_WORDS, 0u);
+    std::vector<float> packed(d->numQuadVals + 64, 0.0f);
+    int rc = cute_quad_pack(d->M, rowPtr, cols, vals, d->quadRows, d->qgp.data(), d->qValBase.data(), d->qrecsHost.data(), packed.data());
+    if (rc == CUTE_OK) rc = upload(&d->dQRecs, d->qrecsHost.data(), d->qrecsHost.size());
+    if (rc == CUTE_OK) rc = upload(&d->dQVals, packed.data(), packed.size());
+    if (rc == CUTE_OK) {
+        d->bytes += d->qrecsHost.size() * 4 + packed.size() * 4;
+        d->haveQuads = true;
+    }
+    return rc;
+}
+
+// A layout the upload did not build: made from the device copy of the CSR arrays (the host arrays the
+// format borrowed may be gone by now).  which: 1 brick tiles, 2 quad lists.
+int ensure_layout(const cute_hrpb_dev *cd, int which)
+{
+    cute_hrpb_dev *d = const_cast<cute_hrpb_dev *>(cd);
+    std::lock_guard<std::mutex> guard(d->lock);
+    if (which == 1 ? d->haveBricks : d->haveQuads) return CUTE_OK;
+    std::vector<uint32_t> rowPtr(size_t(d->M) + 1), cols(std::max<uint32_t>(d->nnz, 1u));
+    std::vector<float> vals(std::max<uint32_t>(d->nnz, 1u));
+    HIP_TRY(hipMemcpy(rowPtr.data(), d->dRowPtr, rowPtr.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    if (d->nnz) {
+        HIP_TRY(hipMemcpy(cols.data(), d->dCols, size_t(d->nnz) * sizeof(uint32_t), hipMemcpyDeviceToHost));
+        HIP_TRY(hipMemcpy(vals.data(), d->dCsrVals, size_t(d->nnz) * sizeof(float), hipMemcpyDeviceToHost));
+    }
+    if (which == 2) return build_quads(d, rowPtr.data(), cols.data(), vals.data());
+    cute_hrpb_host h;
+    int rc = cute_hrpb_build(d->M, d->K, rowPtr.data(), cols.data(), vals.data(), &h);
+    if (rc == CUTE_OK) rc = build_bricks(d, &h);
+    cute_hrpb_host_release(&h);
+    return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
 int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_dev **out)
 {
     if (!h || !out || !h->rowPtr || quad_layout < 0 || quad_layout > 2) return CUTE_ERR_ARG;
     *out = nullptr;
     const DeviceContext &c = context();
     if (c.status != CUTE_OK) return c.status;
-    cute_hrpb_tiled t;
-    int rc = cute_hrpb_retile(h, &t);
-    if (rc != CUTE_OK) return rc;
     cute_hrpb_dev *d = new cute_hrpb_dev;
     d->M = h->M;
     d->K = h->K;
     d->nnz = h->nnz;
     d->P = h->numRowPanels;
     d->nb = h->numBlocks;
-    d->numVals = t.numVals;
+    d->numVals = h->nnz;                     // the brick tiles store every entry of the matrix once
     d->brp.assign(h->blockedRowPtr, h->blockedRowPtr + h->numRowPanels + 1);
     d->panelNnz.resize(d->P);
     d->panelCols.resize(d->P);
@@ -265,75 +340,65 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
         uint32_t longest = 0;
         for (uint32_t r = p * CUTE_TM; r < (p + 1) * CUTE_TM; ++r) longest = std::max(longest, h->rowPtr[r + 1] - h->rowPtr[r]);
         d->panelMaxRow[p] = longest;
+        // active columns: the panel's list is ascending and zero-padded to whole blocks
         const uint32_t nblk = d->brp[p + 1] - d->brp[p];
         uint32_t live = 0;
         if (nblk) {
-            const uint32_t *hd = t.hdr + uint64_t(d->brp[p + 1] - 1) * CUTE_TILED_HDR_WORDS;
-            for (uint32_t j = 0; j < 4; ++j) {
-                uint64_t bm;
-                std::memcpy(&bm, hd + 16 + 2 * j, 8);
-                for (uint32_t k = 0; k < 4; ++k) live += ((bm >> (16 * k)) & 0xFFFFull) ? 1u : 0u;
-            }
-            live += (nblk - 1) * CUTE_TK;
+            const uint32_t *last = h->activeCols + uint64_t(d->brp[p + 1] - 1) * CUTE_TK;
+            uint32_t used = CUTE_TK;
+            while (used > 1 && last[used - 1] == 0) --used;
+            live = (nblk - 1) * CUTE_TK + used;
         }
         d->panelCols[p] = live;
     }
-    rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
-    if (rc == CUTE_OK) {
-        // one wavefront of zero padding behind the values: the brick kernel loads A operands
-        // unconditionally at (brick offset + lane rank)
-        std::vector<float> padded(t.numVals + 64, 0.0f);
-        if (t.numVals) std::memcpy(padded.data(), t.vals, t.numVals * sizeof(float));
-        rc = upload(&d->dVals, padded.data(), padded.size());
-    }
-    if (rc == CUTE_OK) rc = upload(&d->dRowPtr, h->rowPtr, uint64_t(h->M) + 1);
+    int rc = upload(&d->dRowPtr, h->rowPtr, uint64_t(h->M) + 1);
     if (rc == CUTE_OK) rc = upload(&d->dCols, h->cols, h->nnz);
     if (rc == CUTE_OK) rc = upload(&d->dCsrVals, h->vals, h->nnz);
-    d->bytes = uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + t.numVals * 4 + (uint64_t(h->M) + 1) * 4 +
-               uint64_t(h->nnz) * 8;
-    cute_hrpb_tiled_release(&t);
+    d->bytes = (uint64_t(h->M) + 1) * 4 + uint64_t(h->nnz) * 8;
+    // Sizes of the quad lists from one sweep over the strips.  Lockstep lists unless they would be mostly padding
+    // (a few very long rows stretch the lists of their panel neighbours): then one list per 4-row strip.
+    const uint32_t S = d->M / 4;
+    std::vector<uint32_t> strip_pairs(S), strip_vals(S);
+    if (rc == CUTE_OK) rc = cute_quad_census(h->M, h->rowPtr, h->cols, h->vals, strip_pairs.data(), strip_vals.data());
     if (rc == CUTE_OK) {
-        // Lockstep lists unless they would be mostly padding (a few very long rows stretch the
-        // lists of their neighbours): then one list per 4-row strip.
-        cute_quad_lists ql;
-        if (quad_layout == 0) {
-            uint64_t groups = 0, pairs = 0;
-            rc = cute_quad_fill(h->M, h->rowPtr, h->cols, &groups, &pairs);
-            quad_layout = (groups && double(pairs) < 0.6 * 16.0 * double(groups)) ? 2 : 1;
+        uint64_t pairs = 0, lock_groups = 0;
+        for (uint32_t p = 0; p < d->P; ++p) {
+            uint32_t longest = 0;
+            for (uint32_t l = 0; l < 4; ++l) { longest = std::max(longest, strip_pairs[4 * p + l]); pairs += strip_pairs[4 * p + l]; }
+            lock_groups += (longest + 3) / 4;
         }
-        if (rc == CUTE_OK)
-            rc = quad_layout == 2 ? cute_quad_build_strips(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql)
-                                  : cute_quad_build(h->M, h->K, h->rowPtr, h->cols, h->vals, &ql);
-        if (rc == CUTE_OK) {
-            d->numGroups = ql.numGroups;
-            d->quadRows = ql.rowsPerList;
-            d->quadPairs = ql.numPairs;
-            d->qgp.assign(ql.groupPtr, ql.groupPtr + ql.numRowPanels + 1);
-            // Device form of the lists: per group a record {16 columns, 64-bit mask of its occupied value
-            // slots, position of its first stored value, pad} and only the occupied slots' values -- slots of
-            // padding pairs and of rows a column does not touch hold zeros and are not stored.
-            std::vector<uint32_t> recs(ql.numGroups * cute_dev::kQuadRecordWords, 0u);
-            std::vector<float> packed;
-            packed.reserve(h->nnz + 64);
-            for (uint64_t g = 0; g < ql.numGroups; ++g) {
-                uint32_t *rec = recs.data() + g * cute_dev::kQuadRecordWords;
-                std::memcpy(rec, ql.cols + g * 16, 16 * sizeof(uint32_t));
-                uint64_t mask = 0;
-                rec[18] = uint32_t(packed.size());
-                for (uint32_t l = 0; l < 64; ++l) {
-                    const float v = ql.vals[g * 64 + l];
-                    if (v != 0.0f) { mask |= 1ull << l; packed.push_back(v); }
-                }
-                rec[16] = uint32_t(mask);
-                rec[17] = uint32_t(mask >> 32);
-            }
-            d->numQuadVals = packed.size();
-            packed.resize(packed.size() + 64, 0.0f);
-            rc = upload(&d->dQRecs, recs.data(), recs.size());
-            if (rc == CUTE_OK) rc = upload(&d->dQVals, packed.data(), packed.size());
-            d->bytes += recs.size() * 4 + packed.size() * 4;
-            cute_quad_release(&ql);
+        if (quad_layout == 0) quad_layout = (lock_groups && double(pairs) < 0.6 * 16.0 * double(lock_groups)) ? 2 : 1;
+        d->quadRows = quad_layout == 2 ? 4u : CUTE_TM;
+        d->quadPairs = pairs;
+        const uint32_t per_unit = d->quadRows / 4, U = S / per_unit;
+        d->qgp.assign(size_t(U) + 1, 0u);
+        d->qValBase.assign(size_t(U) + 1, 0u);
+        uint64_t groups = 0, stored = 0;
+        for (uint32_t u = 0; u < U && rc == CUTE_OK; ++u) {
+            uint32_t longest = 0;
+            d->qValBase[u] = stored;
+            for (uint32_t l = 0; l < per_unit; ++l) { longest = std::max(longest, strip_pairs[u * per_unit + l]); stored += strip_vals[u * per_unit + l]; }
+            groups += per_unit == 4 ? (longest + 3) / 4 : (longest + 15) / 16;
+            if (groups > 0xffffffffull / 64) rc = CUTE_ERR_SHAPE;
+            d->qgp[u + 1] = uint32_t(groups);
         }
+        d->qValBase[U] = stored;
+        d->numGroups = groups;
+        d->numQuadVals = stored;
+    }
+    if (rc == CUTE_OK) {
+        // Which MFMA layout would the planner's default rules use (see cute_spmm_plan_create)?  Build that one now.
+        const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
+        uint64_t slots = 0, bricks = 0;
+        for (uint32_t q = 0; q < d->P; ++q) {
+            if (d->brp[q + 1] == d->brp[q]) continue;
+            const uint32_t list_slots = (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
+            const uint32_t fetches = std::max(d->panelCols[q], list_slots);
+            if (float(d->panelNnz[q]) < kMinReuse * float(fetches) && d->panelMaxRow[q] <= kMaxRowForRows) continue;   // row kernel
+            slots += list_slots;
+            bricks += (d->panelCols[q] + 3u) / 4u;
+        }
+        if (bricks) rc = slots < kSlotsPerBrick * bricks ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
     }
     if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
     *out = d;
@@ -382,8 +447,8 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (tn) t = *tn;
     if (t.path < CUTE_PATH_AUTO || t.path > CUTE_PATH_ROWS) return CUTE_ERR_ARG;
     if (t.precision != CUTE_PREC_FP32 && t.precision != CUTE_PREC_BF16X3) return CUTE_ERR_ARG;
-    const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : 1.25f;
-    const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : 48;   // measured: longer rows serialise a lane group
+    const float min_reuse = t.min_reuse > 0.0f ? t.min_reuse : kMinReuse;
+    const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : kMaxRowForRows;
     // An MFMA work item always spans 64 output columns; when N is narrower the row kernel wastes
     // less, so the reuse a panel must offer to earn the MFMA kernel grows (measured on N = 8..32).
     const float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
@@ -459,7 +524,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
                 slots += uint64_t(d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
                 bricks += (d->panelCols[q] + 3u) / 4u;
             }
-        p->shape = slots < 8u * bricks ? 2 : 1;
+        p->shape = slots < kSlotsPerBrick * bricks ? 2 : 1;
     }
     if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
     // bf16x3 exists for the rolling brick kernel with four columns per lane; any other shape computes in fp32
@@ -634,15 +699,21 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (t.chunk_order != 1 && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
         p->info.dealtChunks = deal_chunks(chunks, num_slabs, uint32_t(c.num_cus) / cute_dev::kNumXcd,
                                           p->shape == 2 || p->ng == 1 ? 8u : 4u, t.chunk_order == 2) ? 1u : 0u;
-    int rc = upload(&p->dChunks, chunks.data(), chunks.size());
+    // the layout this plan's MFMA kernel reads, if the upload has not built it
+    int rc = chunks.empty() ? int(CUTE_OK) : ensure_layout(d, p->shape);
+    if (rc == CUTE_OK) rc = upload(&p->dChunks, chunks.data(), chunks.size());
     if (rc == CUTE_OK && p->shape == 2 && !chunks.empty()) {
-        const uint64_t words = uint64_t(chunks.size()) * cute_dev::kQuadHeadWords;
-        if (hipMalloc(reinterpret_cast<void **>(&p->dHeads), words * sizeof(uint32_t)) != hipSuccess) rc = CUTE_ERR_NOMEM;
-        else {
-            hipLaunchKernelGGL(cute_dev::build_quad_heads, dim3(uint32_t((words + 255u) / 256u)), dim3(256), 0, nullptr, p->dChunks,
-                               uint32_t(chunks.size()), d->dQRecs, p->dHeads);
-            if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) rc = CUTE_ERR_HIP;
+        // one 128-byte head per work item: its descriptor and a copy of its first group's record, so that a
+        // wavefront can ask for its first B rows after one scalar fetch instead of two dependent ones
+        std::vector<uint32_t> heads(chunks.size() * size_t(cute_dev::kQuadHeadWords), 0u);
+        for (size_t i = 0; i < chunks.size(); ++i) {
+            uint32_t *hd = heads.data() + i * cute_dev::kQuadHeadWords;
+            hd[0] = chunks[i].x; hd[1] = chunks[i].y; hd[2] = chunks[i].z; hd[3] = chunks[i].w;
+            if (chunks[i].x < chunks[i].y)               // an empty chunk (a strip without pairs) keeps a zero record
+                std::memcpy(hd + 4, d->qrecsHost.data() + size_t(chunks[i].x) * cute_dev::kQuadRecordWords,
+                            cute_dev::kQuadRecordWords * sizeof(uint32_t));
         }
+        rc = upload(&p->dHeads, heads.data(), heads.size());
     }
     if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
     p->unitRows = CUTE_TM / upp;

@@ -149,6 +149,80 @@ int cute_quad_build(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32
     return CUTE_OK;
 }
 
+// What the two layouts would hold, without building either: for every 4-row strip the length of its
+// merged column list (pairs) and the number of values it stores (nonzero entries; an explicit zero in
+// the input is an empty slot).  Group counts, padding and the fill of either layout follow from these.
+int cute_quad_census(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t *stripPairs,
+                     uint32_t *stripVals)
+{
+    if (!rowPtr || !stripPairs || !stripVals || (rowPtr[M] && (!cols || !vals))) return CUTE_ERR_ARG;
+    const uint32_t S = (M + 3) / 4;
+    cute::parallel_ranges(S, 1024, [&](uint64_t b, uint64_t e, unsigned) {
+        for (uint64_t q = b; q < e; ++q) {
+            uint32_t stored = 0;
+            stripPairs[q] = merge_row_group(M, rowPtr, cols, vals, uint32_t(q) * 4, [&](uint32_t, const float *v) {
+                for (int i = 0; i < 4; ++i) stored += v[i] != 0.0f;
+            });
+            stripVals[q] = stored;
+        }
+    });
+    return CUTE_OK;
+}
+
+// The device form of the lists, written directly: per group a record of CUTE_QUAD_RECORD_WORDS words
+// {16 columns, 64-bit mask of the occupied value slots (slot 4p+i = pair p, row i), index of the group's
+// first stored value, pad} and the stored values of all groups in slot order.  rowsPerList 16: four
+// lockstep lists per panel (unit = panel), 4: one list per strip (unit = strip).  groupPtr[U+1] and
+// valBase[U] (index of each unit's first stored value) come from cute_quad_census; recs has
+// groupPtr[U] * CUTE_QUAD_RECORD_WORDS words, packed valBase[U-1] + (values of the last unit) floats.
+int cute_quad_pack(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t rowsPerList,
+                   const uint32_t *groupPtr, const uint64_t *valBase, uint32_t *recs, float *packed)
+{
+    if (!rowPtr || !groupPtr || !valBase || !recs || !packed || (rowPtr[M] && (!cols || !vals))) return CUTE_ERR_ARG;
+    if (rowsPerList != 16 && rowsPerList != 4) return CUTE_ERR_ARG;
+    const uint32_t lists = rowsPerList / 4;                       // lists that advance together in one unit
+    const uint32_t U = (M + rowsPerList - 1) / rowsPerList;
+    cute::parallel_ranges(U, 64, [&](uint64_t b, uint64_t e, unsigned) {
+        struct Pair { uint32_t col; float v[4]; };
+        std::vector<Pair> list[4];
+        for (uint64_t u = b; u < e; ++u) {
+            for (uint32_t l = 0; l < lists; ++l) {
+                list[l].clear();
+                merge_row_group(M, rowPtr, cols, vals, uint32_t(u) * rowsPerList + l * 4, [&](uint32_t col, const float *v) {
+                    Pair p;
+                    p.col = col;
+                    std::memcpy(p.v, v, sizeof(p.v));
+                    list[l].push_back(p);
+                });
+            }
+            uint64_t next_val = valBase[u];
+            for (uint64_t g = groupPtr[u]; g < groupPtr[u + 1]; ++g) {
+                uint32_t *rec = recs + g * CUTE_QUAD_RECORD_WORDS;
+                const uint32_t local = uint32_t(g - groupPtr[u]);
+                uint64_t mask = 0;
+                rec[18] = uint32_t(next_val);
+                rec[19] = 0;
+                for (uint32_t p = 0; p < 16; ++p) {
+                    // lockstep: pair p is step p/4 of list p%4; strips: pair p is entry p of the one list
+                    const uint32_t l = lists == 4 ? p % 4 : 0;
+                    const uint32_t step = lists == 4 ? local * 4 + p / 4 : local * 16 + p;
+                    const std::vector<Pair> &src = list[l];
+                    if (step < src.size()) {
+                        rec[p] = src[step].col;
+                        for (uint32_t i = 0; i < 4; ++i)
+                            if (src[step].v[i] != 0.0f) { mask |= 1ull << (4 * p + i); packed[next_val++] = src[step].v[i]; }
+                    } else {
+                        rec[p] = src.empty() ? 0u : src.back().col;        // padding repeats the list's last column
+                    }
+                }
+                rec[16] = uint32_t(mask);
+                rec[17] = uint32_t(mask >> 32);
+            }
+        }
+    });
+    return CUTE_OK;
+}
+
 // The same pairs with one list per 4-row strip instead of four lockstep lists per panel: nothing
 // is padded to a longer neighbour, which is what a matrix with a few very long rows needs (the
 // strip holding such a row would otherwise stretch the other three of its panel).  A group is 16

@@ -11,6 +11,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/cutespmm.h"
+
 namespace cute_dev {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -31,7 +33,7 @@ constexpr int kWaveSize = 64;
 constexpr int kWavesPerGroup = 4;
 constexpr int kHdrWords = 32;
 constexpr int kNumXcd = 8;
-constexpr int kQuadRecordWords = 20;   // device record of one quad-list group: 16 columns, mask lo/hi, first value, pad
+constexpr int kQuadRecordWords = CUTE_QUAD_RECORD_WORDS;   // device record of one quad-list group: 16 columns, mask lo/hi, first value, pad
 constexpr int kQuadHeadWords = 32;     // quad kernels, per chunk: descriptor (4 words), first group's record, padding to 128 bytes
 
 // Work-groups are handed to the 8 XCDs round-robin; this maps the hardware id to a
@@ -695,20 +697,6 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
                 }
         }
     }
-}
-
-// Fills the quad kernels' per-chunk entries from the chunk list and the group records (run once per plan).
-__global__ __launch_bounds__(256) void build_quad_heads(const uint4 *__restrict__ chunks, uint32_t num_chunks,
-                                                        const uint32_t *__restrict__ qrecs, uint32_t *__restrict__ heads)
-{
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= num_chunks * uint32_t(kQuadHeadWords)) return;
-    const uint32_t c = i / uint32_t(kQuadHeadWords), w = i % uint32_t(kQuadHeadWords);
-    const uint4 ck = chunks[c];
-    uint32_t v = 0;                                   // an empty chunk (a strip without pairs) keeps a zero record
-    if (w < 4u) v = w == 0 ? ck.x : w == 1 ? ck.y : w == 2 ? ck.z : ck.w;
-    else if (w < 4u + uint32_t(kQuadRecordWords) && ck.x < ck.y) v = qrecs[size_t(ck.x) * kQuadRecordWords + (w - 4u)];
-    heads[i] = v;
 }
 
 template <bool FULL, bool STRIPS>

@@ -174,6 +174,19 @@ int cute_quad_fill(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, uin
 int cute_quad_build_strips(uint32_t M, uint32_t K, const uint32_t *rowPtr, const uint32_t *cols, const float *vals,
                            cute_quad_lists *out);
 void cute_quad_release(cute_quad_lists *q);
+/* Sizes of either layout without building it: per 4-row strip (there are ceil(M/4)) the length of its
+ * merged column list and the number of values it stores (nonzero entries). */
+int cute_quad_census(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t *stripPairs,
+                     uint32_t *stripVals);
+/* The device form of the lists, written directly from the CSR matrix (what cute_hrpb_upload sends): per
+ * group a record of CUTE_QUAD_RECORD_WORDS words {16 columns, 64-bit mask of the occupied value slots
+ * (slot 4p+i = pair p, row i), index of the group's first stored value, 0} and, in `packed`, the stored
+ * (nonzero) values of all groups in slot order.  rowsPerList 16: lockstep lists, a unit is a panel;
+ * 4: a unit is a strip.  groupPtr[U+1] and valBase[U] (index of each unit's first stored value) follow
+ * from cute_quad_census. */
+#define CUTE_QUAD_RECORD_WORDS 20u
+int cute_quad_pack(uint32_t M, const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t rowsPerList,
+                   const uint32_t *groupPtr, const uint64_t *valBase, uint32_t *recs, float *packed);
 
 /* ------------------------------------------------------------------------------------
  * host: launch partition.            Replaces SPMM_TC::partition (spmm.cu:776-812).

@@ -129,3 +129,36 @@ def test_lockstep_tail_and_pair_count(cs):
     assert cs.load_library().cute_quad_fill(M, rp32.ctypes.data_as(C.POINTER(C.c_uint32)), cl32.ctypes.data_as(C.POINTER(C.c_uint32)),
                                             C.byref(g), C.byref(n)) == 0
     assert (g.value, n.value) == (q["numGroups"], pairs)
+
+
+def test_direct_packing_equals_packing_the_lists(cs):
+    """cute_quad_pack (what the upload sends to the device, written straight from the CSR matrix) against the
+    same records made here from the inspectable host form of the lists: per group 16 columns, the mask of
+    nonzero value slots, the running index of the first stored value, and the stored values in slot order."""
+    rng = np.random.default_rng(31)
+    cases = [(64, 96, dict(density=0.1)), (32, 64, dict(row_nnz=0)), (48, 2048, dict(row_nnz=lambda r: 900 if r == 3 else 5)),
+             (160, 64, dict(density=0.4, empty_rows=set(range(16, 40))))]
+    for M, K, kw in cases:
+        rp, cl, vl = random_csr(rng, M, K, **kw)
+        if len(vl) > 4:
+            vl[rng.choice(len(vl), 3, replace=False)] = 0.0          # explicit zeros are empty slots, not stored values
+        for strips in (False, True):
+            q = cs.quad_lists(M, K, rp, cl, vl, strips=strips)
+            got = cs.quad_pack(M, rp, cl, vl, strips=strips)
+            assert np.array_equal(got["groupPtr"], q["groupPtr"])
+            G = q["numGroups"]
+            recs = np.zeros((G, 20), np.uint32)
+            packed = []
+            for g in range(G):
+                recs[g, :16] = q["cols"][g]
+                recs[g, 18] = len(packed)
+                mask = 0
+                for slot in range(64):
+                    v = q["vals"][g, slot]
+                    if v != 0.0:
+                        mask |= 1 << slot
+                        packed.append(v)
+                recs[g, 16], recs[g, 17] = mask & 0xFFFFFFFF, mask >> 32
+            assert np.array_equal(got["recs"], recs), (M, K, strips)
+            assert got["packed"].tobytes() == np.asarray(packed, np.float32).tobytes(), (M, K, strips)
+            assert int(got["stripPairs"].sum()) == q["numPairs"] and int(got["stripVals"].sum()) == len(packed)
