@@ -29,15 +29,38 @@ def algorithmic_bytes(M, K, N, nnz):
     return nnz * 8 + (M + 1) * 4 + K * N * 4 + M * N * 4
 
 
-def recorded_traffic(workload):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), if a
-    record for this workload has been committed under profiles/."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic_%s.json" % workload)
+KERNEL_SOURCES = ("cutespmm_ae_amd/csrc/kernels.hip.hpp", "cutespmm_ae_amd/csrc/device.hip")
+
+
+def kernel_sources_sha16():
+    """Fingerprint of the device code the counters under profiles/ were taken with."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(workload, kernel):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): read from the record
+    committed under profiles/ -- but only if that record was taken with the kernel sources as they are now
+    and for the kernel that ran; otherwise the traffic is unknown (None) and the source says why."""
+    rel = "profiles/hbm_traffic_%s.json" % workload
     try:
-        rec = json.load(open(path)).get(workload)
-        return None if rec is None else float(rec["fetch_bytes"]) + float(rec["write_bytes"])
-    except (OSError, ValueError, KeyError):
-        return None
+        rec = json.load(open(os.path.join(ROOT, rel))).get(workload)
+        total = float(rec["fetch_bytes"]) + float(rec["write_bytes"])
+    except (OSError, ValueError, KeyError, TypeError):
+        return None, None
+    source = dict(file=rel, kernel=rec.get("kernel"), kernel_sources_sha16=rec.get("kernel_sources_sha16"),
+                  recorded_at_commit=rec.get("commit"))
+    if rec.get("kernel_sources_sha16") != kernel_sources_sha16():
+        source["stale"] = "kernel sources changed since the counters were recorded"
+        return None, source
+    if kernel and rec.get("kernel") and not str(rec["kernel"]).startswith(kernel):
+        source["stale"] = "recorded for another kernel"
+        return None, source
+    return total, source
 
 
 def cpu_baseline(A, B, budget_s=10.0):
@@ -82,6 +105,9 @@ def main():
     ap.add_argument("--path", choices=("auto", "mfma", "rows"), default="auto", help="kernel family (default: the planner's choice)")
     ap.add_argument("--mfma-shape", type=int, default=0, help="1: 16x16x4 brick kernel, 2: 4x4x1 quad kernel, 0: planner's choice")
     ap.add_argument("--pipeline", type=int, default=0, help="brick kernel variant: 1 rolling, 2 pipelined, 0: default")
+    ap.add_argument("--precision", choices=("fp32", "bf16x3"), default="fp32",
+                    help="bf16x3: the brick kernel on the bf16 matrix pipeline (opt-in, error below 2^-15); default fp32")
+    ap.add_argument("--no-csr", action="store_true", help="skip the three plain CSR comparison kernels")
     ap.add_argument("--chunk-order", type=int, default=0,
                     help="MFMA work items: 0 planner's choice, 1 panel order, 2 dealt to the SIMDs longest first")
     ap.add_argument("--graph", action="store_true",
@@ -113,7 +139,8 @@ def main():
     dB = torch.from_numpy(B).cuda()
     dC = torch.empty((A.M, N), device="cuda")
     plan = cs.SPMM_TC(h, N, path={"auto": cs.PATH_AUTO, "mfma": cs.PATH_BRICK, "rows": cs.PATH_ROWS}[args.path],
-                      mfma_shape=args.mfma_shape, pipeline=args.pipeline, chunk_order=args.chunk_order)
+                      mfma_shape=args.mfma_shape, pipeline=args.pipeline, chunk_order=args.chunk_order,
+                      precision=cs.PREC_BF16X3 if args.precision == "bf16x3" else cs.PREC_FP32)
     stream = torch.cuda.current_stream()
 
     ramp_end = time.perf_counter() + args.ramp_ms * 1e-3
@@ -164,14 +191,17 @@ def main():
         kernels.append("csr_rows_batched")
     if plan.info["numAtomicChunks"]:
         kernels.append("reduce_partials")
+    dominant = plan.kernel_name if plan.info["numChunks"] else "csr_rows_batched"
+    traffic, traffic_source = recorded_traffic(cfg["name"], dominant)
     roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                    traffic=recorded_traffic(cfg["name"]), kernel=plan.kernel_name if plan.info["numChunks"] else "csr_rows_batched",
+                    traffic=traffic, traffic_source=traffic_source, kernel=dominant,
                     kernels_per_step=kernels, kernel_ms=kernel_ms, kernel_ms_single_bracketed_median=float(np.median(each)),
                     algorithmic_bytes=abytes)
 
     out = dict(metric="SpMM GFLOP/s (2*nnz*N/t) on 1 MI355X", value=value, unit="GFLOP/s", n_gpus=1,
                steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
-               scaling="weak", vs_baseline=None, dtype="f32", data="synthetic (seeded generator)",
+               scaling="weak", vs_baseline=None, dtype="f32" if plan.info["precision"] == cs.PREC_FP32 else "bf16x3 (f32 accumulate)",
+               data="synthetic (seeded generator)",
                launch="hip graph replay" if args.graph else "stream launches", ramp_ms=args.ramp_ms,
                config=dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, blocks=h.numBlocks,
                            bricks=h.num_bricks, plan={k: plan.info[k] for k in
@@ -179,12 +209,27 @@ def main():
                                                        "numBrickPanels", "numRowPanelsSparse", "dealtChunks")}),
                roofline=roofline)
 
+    if not args.no_csr:
+        # the plain CSR kernels on the same inputs and clocks: the "best simple CSR kernel" a caller would write instead
+        csr_us = {}
+        for alg, name in ((0, "thread_per_element"), (1, "wave_per_row_scalar"), (2, "wave_per_row_vector")):
+            iters = 30 if A.nnz < 10_000_000 else 5
+            t = cs.csr_spmm_time(alg, h, dB, dC, warmup=3, iters=iters, stream=stream)
+            csr_us[name] = float(np.median(t)) * 1e3
+        best = min(csr_us.values())
+        out["simple_csr_kernels_us"] = csr_us
+        out["speedup_over_best_simple_csr"] = best / (float(np.median(each)) * 1e3)     # both timed one launch per event pair
+        plan.run(dB, dC)                                # the output checked below is the planned path's
+        torch.cuda.synchronize()
+
     ref = None
     if not args.no_cpu:
         out["cpu_baseline"], ref = cpu_baseline(A, B)
         got = dC.cpu().numpy()
         out["backward_error_vs_oracle"] = cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, got)
         out["reference_metric_vs_oracle"] = cs.check_gemm_correctness_coo(ref, got)
+        out["parity_note"] = ("checked against this build's CPU oracle (inc.h:71-83 restated); the reference's own comparison path, "
+                              "cuSPARSE CSR SpMM (spmm.cu:912-938), is a closed binary with no stored outputs: parity with its bits is unpinned")
 
     if args.detail:
         detail = dict(workload=cfg["name"], paths={}, csr={})

@@ -18,6 +18,15 @@ thread_local std::string g_hip_error;
 constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
 constexpr uint32_t kMaxRowForRows = 48;     // ... unless it holds a row longer than this: one lane group would serialise it
 constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
+// B and C together larger than the Infinity Cache: whatever the caller does between launches, their rows come
+// from HBM.  There the brick kernel's wider row pieces (16 lanes x 16 bytes per row and column group, two groups
+// per wavefront from N = 128 on) beat the quad kernel's 256-byte pieces by 20-25 % (9-point stencils of 0.25 to
+// 1 million rows) -- as long as its matrix work, 32 cycles per brick and 16 columns however empty the brick,
+// stays below the time the operands take to stream at 4 TB/s; on R-MAT graphs, where it is 1.4 to 1.7 times
+// that, the two kernels are within 10 % of each other either way and the rule above keeps deciding.  While the
+// operands fit the cache the quad kernel is level or ahead.
+constexpr uint64_t kInfinityCacheBytes = 256ull << 20;
+constexpr double kStreamBytesPerSecond = 4.0e12, kSimdCyclesPerSecond = 1024 * 2.4e9, kCyclesPerBrickTile = 32.0;
 
 inline int hip_fail(hipError_t e, const char *what, int line)
 {
@@ -398,7 +407,11 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
             slots += list_slots;
             bricks += (d->panelCols[q] + 3u) / 4u;
         }
-        if (bricks) rc = slots < kSlotsPerBrick * bricks ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
+        // (the width is not known yet: 128 columns stand in for it in the rule for operands beyond the cache)
+        const bool beyond_cache = (uint64_t(d->K) + d->M) * 128u * sizeof(float) > kInfinityCacheBytes &&
+                                  double(bricks) * 8.0 * kCyclesPerBrickTile / kSimdCyclesPerSecond <=
+                                      (double(uint64_t(d->K) + d->M) * 512.0 + double(d->nnz) * 8.0) / kStreamBytesPerSecond;
+        if (bricks) rc = (slots < kSlotsPerBrick * bricks && !beyond_cache) ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
     }
     if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
     *out = d;
@@ -498,7 +511,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // column group per lane halves the registers and doubles the resident wavefronts; the same when the row blocks
     // are the larger part of the launch anyway (ted_B, N = 128).
     bool ng_for_mixed = false;
-    if (p->ng == 2 && t.brick_groups == 0 && n_brick && n_rows) {
+    // (not when B and C come from HBM: there the wider row pieces of two column groups count for more)
+    const bool beyond_cache = (uint64_t(d->K) + d->M) * N * sizeof(float) > kInfinityCacheBytes;
+    if (p->ng == 2 && t.brick_groups == 0 && n_brick && n_rows && !beyond_cache) {
         const uint64_t row_blocks = (uint64_t(n_rows) * CUTE_TM * p->rows_slabs + (256u >> p->rows_logl) - 1) / (256u >> p->rows_logl);
         const uint64_t groups = (uint64_t(n_brick) * ((N + 127u) / 128u) + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
         if (row_blocks + groups > uint64_t(c.num_cus) * 4u || row_blocks >= groups) { p->ng = 1; ng_for_mixed = true; }
@@ -525,6 +540,11 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
                 bricks += (d->panelCols[q] + 3u) / 4u;
             }
         p->shape = slots < kSlotsPerBrick * bricks ? 2 : 1;
+        if (beyond_cache) {
+            const double matrix_s = double(bricks) * double((N + 15u) / 16u) * kCyclesPerBrickTile / kSimdCyclesPerSecond;
+            const double stream_s = (double(uint64_t(d->K) + d->M) * N * 4.0 + double(d->nnz) * 8.0) / kStreamBytesPerSecond;
+            if (matrix_s <= stream_s) p->shape = 1;
+        }
     }
     if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
     // bf16x3 exists for the rolling brick kernel with four columns per lane; any other shape computes in fp32

@@ -330,8 +330,10 @@ float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, cons
 
 /* ------------------------------------------------------------------------------------
  * device: upload.        Replaces the cudaMalloc/cudaMemcpy tail of DATASTRUCT
- * (data.cu:327-334) and HRPB::freeDevice (data.cu:336-339).  Uploads the MFMA-tiled
- * layout, the per-panel descriptors and the borrowed CSR (for the sparse-panel path).
+ * (data.cu:327-334) and HRPB::freeDevice (data.cu:336-339).  Uploads the CSR arrays (the row
+ * kernel's input) and the one MFMA layout the planner's default rules would use for this matrix --
+ * brick tiles or quad lists, or neither if every panel would go to the row kernel; a plan that asks
+ * for the other layout builds it then, from the device copy of the CSR arrays.
  * ---------------------------------------------------------------------------------- */
 typedef struct cute_hrpb_dev cute_hrpb_dev;
 int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out);
@@ -392,6 +394,8 @@ typedef struct cute_plan_info {
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;
+/* Plan creation copies its tables to the device with synchronous copies (and, if the plan is the first to
+ * need an MFMA layout the upload did not build, builds that layout): call it outside stream capture. */
 int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunables *t /* may be NULL */,
                           cute_spmm_plan **out);
 int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out);
@@ -401,7 +405,13 @@ void cute_spmm_plan_free(cute_spmm_plan *p);
  * need not zero it (the reference requires cudaMemset first, run.cu:43,49).  No atomics are
  * used, so equal inputs give equal bits.  A plan whose panels were cut (numAtomicChunks > 0)
  * keeps their partial tiles in a buffer of its own: launches of ONE plan must not overlap in
- * time (same stream, or ordered by events); different plans are independent. */
+ * time (same stream, or ordered by events); different plans are independent.
+ * B must be finite for the MFMA kernels to give the CSR product: like the reference's kernel
+ * (kernel.cu:26-27,149) they multiply a stored zero into a real B row wherever a brick or a list slot
+ * has no entry, so an Inf or NaN in a B row turns into NaN in every row of C whose panel (brick kernels:
+ * 16 rows; quad kernels: the 4-row group) has that column active, and one in B row 0 reaches every panel
+ * that pads its last block.  Rows the planner sends to the row kernel only see the B rows they reference.
+ * A caller whose B may hold Inf or NaN plans with path = CUTE_PATH_ROWS, which is exact in that sense. */
 int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
 
 /* cute_spmm_run for callers that cannot allocate device memory (code under HIP graph capture, serving

@@ -238,6 +238,41 @@ def test_bf16x3_precision_path(cs, orc, torch_cuda):
         cs.SPMM_TC(h, N, precision=2)
 
 
+def test_non_finite_b_rows(cs, torch_cuda):
+    """What an Inf in B does, path by path.  The row kernel is exact: only rows of C that reference the B row see it.
+    The MFMA kernels multiply stored zeros into real B rows (as the reference's kernel does, kernel.cu:26-27,149):
+    the Inf spreads as NaN over the rows that share a panel (brick kernels) or a 4-row group (quad kernels) with a
+    row that references it -- never further -- and an Inf in B row 0 reaches every panel that pads its last block."""
+    rng = np.random.default_rng(5)
+    M, K, N = 64, 128, 64
+    # three entries per row, none in column 0, column 77 referenced by row 21 only
+    pool = np.array([c for c in range(1, K) if c != 77])
+    cols = [np.sort(rng.choice(pool, 3, replace=False)) for _ in range(M)]
+    cols[21] = np.sort(np.append(rng.choice(pool, 2, replace=False), 77))
+    rp2 = (3 * np.arange(M + 1)).astype(np.uint32)
+    cl2 = np.concatenate(cols).astype(np.uint32)
+    vl2 = rng.standard_normal(3 * M).astype(np.float32)
+    h = cs.HRPB(M, K, rp2, cl2, vl2)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    B[77, 5] = np.inf
+    out, _ = _run(cs, torch_cuda, h, B, path=cs.PATH_ROWS)
+    bad = ~np.isfinite(out)
+    assert bad[21, 5] and bad.sum() == 1
+    for name, kw, rows_hit in (("brick", dict(path=cs.PATH_BRICK, mfma_shape=1), range(16, 32)),
+                               ("brick_pipelined", dict(path=cs.PATH_BRICK, mfma_shape=1, pipeline=2), range(16, 32)),
+                               ("quad", dict(path=cs.PATH_BRICK, mfma_shape=2), range(20, 24))):
+        out, _ = _run(cs, torch_cuda, h, B, **kw)
+        bad = ~np.isfinite(out)
+        assert bad[21, 5] and set(np.nonzero(bad.any(1))[0]) <= set(rows_hit) and not bad[:, :5].any() and not bad[:, 6:].any(), name
+    # B row 0 is what padding slots point at
+    B[77, 5] = 1.0
+    B[0, 9] = np.inf
+    out, _ = _run(cs, torch_cuda, h, B, path=cs.PATH_ROWS)
+    assert np.isfinite(out).all()                                  # no row references column 0
+    out, _ = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=1)
+    assert not np.isfinite(out[:, 9]).all() and np.isfinite(np.delete(out, 9, axis=1)).all()
+
+
 def test_edge_shapes(cs, orc, torch_cuda):
     from test_oracle_pins import _edge_cases
     rng = np.random.default_rng(0)
