@@ -91,6 +91,54 @@ def cpu_baseline(A, B, budget_s=10.0):
     return res, out
 
 
+INFINITY_CACHE_BYTES = 256 << 20
+
+
+def hbm_fed_leg(torch, cs, plan, h, dB, dC, N, set_bytes, abytes, flops, steps):
+    """The same launches over enough rotating (B, C) buffer sets that no cache can hold them (1.25 GB, five times
+    the Infinity Cache): every B row then comes from HBM and every C row goes there.  The main measurement
+    re-runs one set; when that set fits the 256 MB Infinity Cache, the cache serves most of it."""
+    if set_bytes > INFINITY_CACHE_BYTES:
+        return dict(sets=1, note="one set of B and C (%.0f MB) already exceeds the Infinity Cache: the main measurement is HBM-fed"
+                                 % (set_bytes / 1e6))
+    sets = max(2, -(-5 * INFINITY_CACHE_BYTES // set_bytes))
+    dBs = [dB] + [dB.clone() for _ in range(sets - 1)]
+    dCs = [dC] + [torch.empty_like(dC) for _ in range(sets - 1)]
+
+    def timed(p):
+        i = 0
+        for _ in range(max(sets, 50)):
+            p.run(dBs[i % sets], dCs[i % sets]); i += 1
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            p.run(dBs[i % sets], dCs[i % sets]); i += 1
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+    ms, kernel_ms = timed(plan)
+    res = dict(sets=sets, bytes_cycled=sets * set_bytes, steps=steps, ms_per_step=ms, kernel_ms=kernel_ms,
+               value=flops / (ms * 1e-3) / 1e9, unit="GFLOP/s", achieved_GBps=abytes / (kernel_ms * 1e-3) / 1e9,
+               frac=abytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, kernel=plan.kernel_name)
+    if plan.info["numChunks"]:
+        # either MFMA kernel forced, under the same conditions: the planner's choice assumes nothing about residency
+        alt = {}
+        for name, shape in (("quad", 2), ("brick", 1)):
+            alt[name] = timed(cs.SPMM_TC(h, N, mfma_shape=shape))[1] * 1e3
+        res["mfma_kernels_forced_us"] = alt
+        # the planner told that its operands come from HBM (cute_tunables.operand_residency = 1); by default it goes by size
+        told = cs.SPMM_TC(h, N, operand_residency=1)
+        t_ms, t_kernel_ms = timed(told)
+        res["planner_told_operands_are_cold"] = dict(kernel=told.kernel_name, ms_per_step=t_ms, value=flops / (t_ms * 1e-3) / 1e9,
+                                                     frac=abytes / (t_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+    plan.run(dB, dC)
+    torch.cuda.synchronize()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +156,11 @@ def main():
     ap.add_argument("--precision", choices=("fp32", "bf16x3"), default="fp32",
                     help="bf16x3: the brick kernel on the bf16 matrix pipeline (opt-in, error below 2^-15); default fp32")
     ap.add_argument("--no-csr", action="store_true", help="skip the three plain CSR comparison kernels")
+    ap.add_argument("--rotate", type=int, default=1,
+                    help="number of (B, C) buffer sets the timed steps cycle through (default 1: the same buffers every step, "
+                         "which the 256 MB Infinity Cache then serves when they fit it)")
+    ap.add_argument("--no-hbm-leg", action="store_true",
+                    help="skip the second measurement over enough rotating buffer sets to exceed the Infinity Cache")
     ap.add_argument("--chunk-order", type=int, default=0,
                     help="MFMA work items: 0 planner's choice, 1 panel order, 2 dealt to the SIMDs longest first")
     ap.add_argument("--graph", action="store_true",
@@ -138,6 +191,10 @@ def main():
     h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
     dB = torch.from_numpy(B).cuda()
     dC = torch.empty((A.M, N), device="cuda")
+    if args.rotate < 1:
+        sys.exit("bench.py: --rotate needs at least one buffer set")
+    dBs = [dB] + [dB.clone() for _ in range(args.rotate - 1)]
+    dCs = [dC] + [torch.empty_like(dC) for _ in range(args.rotate - 1)]
     plan = cs.SPMM_TC(h, N, path={"auto": cs.PATH_AUTO, "mfma": cs.PATH_BRICK, "rows": cs.PATH_ROWS}[args.path],
                       mfma_shape=args.mfma_shape, pipeline=args.pipeline, chunk_order=args.chunk_order,
                       precision=cs.PREC_BF16X3 if args.precision == "bf16x3" else cs.PREC_FP32)
@@ -169,9 +226,12 @@ def main():
     ev0.record(stream)
     if graph is not None:
         graph.replay()
-    else:
+    elif args.rotate == 1:
         for _ in range(args.steps):
             plan.run(dB, dC)
+    else:
+        for i in range(args.steps):
+            plan.run(dBs[i % args.rotate], dCs[i % args.rotate])
     ev1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -202,12 +262,16 @@ def main():
                steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
                scaling="weak", vs_baseline=None, dtype="f32" if plan.info["precision"] == cs.PREC_FP32 else "bf16x3 (f32 accumulate)",
                data="synthetic (seeded generator)",
-               launch="hip graph replay" if args.graph else "stream launches", ramp_ms=args.ramp_ms,
+               launch="hip graph replay" if args.graph else "stream launches", ramp_ms=args.ramp_ms, buffer_sets=args.rotate,
                config=dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, blocks=h.numBlocks,
                            bricks=h.num_bricks, plan={k: plan.info[k] for k in
                                                       ("slabWidth", "numSlabs", "numChunks", "numAtomicChunks",
                                                        "numBrickPanels", "numRowPanelsSparse", "dealtChunks")}),
                roofline=roofline)
+
+    set_bytes = (A.K + A.M) * N * 4
+    if not args.no_hbm_leg and args.rotate == 1 and not args.graph:
+        out["hbm_fed"] = hbm_fed_leg(torch, cs, plan, h, dB, dC, N, set_bytes, abytes, flops, min(args.steps, 500))
 
     if not args.no_csr:
         # the plain CSR kernels on the same inputs and clocks: the "best simple CSR kernel" a caller would write instead

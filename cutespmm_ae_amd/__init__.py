@@ -77,7 +77,7 @@ class cute_quad_lists(C.Structure):
 class cute_tunables(C.Structure):
     _fields_ = [("path", C.c_int32), ("precision", C.c_int32), ("min_reuse", C.c_float), ("slots", C.c_uint32),
                 ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("mfma_shape", C.c_uint32), ("max_row_nnz", C.c_uint32),
-                ("chunk_order", C.c_uint32), ("reserved", C.c_uint32 * 2)]
+                ("chunk_order", C.c_uint32), ("operand_residency", C.c_uint32), ("reserved", C.c_uint32 * 1)]
 
 
 class cute_plan_info(C.Structure):
@@ -560,13 +560,13 @@ class SPMM_TC:
     (spmm.cu:823-839) on torch's current stream.  MatB [K,N], MatC [M,N] float32 GPU tensors."""
 
     def __init__(self, hrpb, N, path=PATH_AUTO, precision=PREC_FP32, min_reuse=0.0, slots=0, max_chunk_blocks=0,
-                 brick_groups=0, pipeline=0, mfma_shape=0, max_row_nnz=0, chunk_order=0):
+                 brick_groups=0, pipeline=0, mfma_shape=0, max_row_nnz=0, chunk_order=0, operand_residency=0):
         self.hrpb = hrpb
         self.M, self.K, self.N = hrpb.M, hrpb.K, int(N)
         self._plan = C.c_void_p()
         t = cute_tunables(path=path, precision=precision, min_reuse=min_reuse, slots=slots,
                           max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline, mfma_shape=mfma_shape,
-                          max_row_nnz=max_row_nnz, chunk_order=chunk_order)
+                          max_row_nnz=max_row_nnz, chunk_order=chunk_order, operand_residency=operand_residency)
         _check(load_library().cute_spmm_plan_create(hrpb.upload(), self.N, C.byref(t), C.byref(self._plan)),
                "cute_spmm_plan_create")
         info = cute_plan_info()

@@ -512,7 +512,9 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // are the larger part of the launch anyway (ted_B, N = 128).
     bool ng_for_mixed = false;
     // (not when B and C come from HBM: there the wider row pieces of two column groups count for more)
-    const bool beyond_cache = (uint64_t(d->K) + d->M) * N * sizeof(float) > kInfinityCacheBytes;
+    if (t.operand_residency > 2) { delete p; return CUTE_ERR_ARG; }
+    const bool beyond_cache = t.operand_residency ? t.operand_residency == 1
+                                                  : (uint64_t(d->K) + d->M) * N * sizeof(float) > kInfinityCacheBytes;
     if (p->ng == 2 && t.brick_groups == 0 && n_brick && n_rows && !beyond_cache) {
         const uint64_t row_blocks = (uint64_t(n_rows) * CUTE_TM * p->rows_slabs + (256u >> p->rows_logl) - 1) / (256u >> p->rows_logl);
         const uint64_t groups = (uint64_t(n_brick) * ((N + 127u) / 128u) + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;

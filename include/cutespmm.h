@@ -374,7 +374,10 @@ typedef struct cute_tunables {
     uint32_t chunk_order;      /* MFMA work items: 0 library's choice (a launch that is resident at once: dealt to the SIMDs longest
                                   first where that shortens the fullest SIMD; a larger launch whose longest item is four times the
                                   mean: long items first); 1 always in panel order; 2 always dealt; 3 always long items first */
-    uint32_t reserved[2];
+    uint32_t operand_residency; /* where B and C are when a launch starts: 0 decided by size (from HBM when they exceed the 256 MiB
+                                  Infinity Cache together), 1 from HBM (a product on data no cache holds), 2 cache-resident
+                                  (the same operands again and again).  Chooses between the MFMA kernels, nothing else. */
+    uint32_t reserved[1];
 } cute_tunables;
 
 typedef struct cute_plan_info {

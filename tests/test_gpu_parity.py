@@ -376,6 +376,19 @@ def test_work_items_dealt_by_length(cs, orc, torch_cuda):
     assert plan.info["dealtChunks"] == 0
     with pytest.raises(cs.CuteError):
         cs.SPMM_TC(h2, 64, chunk_order=4)
+    # where the operands live only changes which MFMA kernel runs
+    A5 = cs.gen_config(2, 1 / 16.0)
+    h5 = cs.HRPB(A5.M, A5.K, A5.rowPtr, A5.cols, A5.vals)
+    B5 = rng.standard_normal((A5.K, 128)).astype(np.float32)
+    ref5 = orc.spmm_csr(A5.rowPtr, A5.cols, A5.vals, B5)
+    names = set()
+    for res in (0, 1, 2):
+        out, plan = _run(cs, torch_cuda, h5, B5, operand_residency=res)
+        names.add(plan.kernel_name)
+        assert cs.backward_error(A5.rowPtr, A5.cols, A5.vals, B5, ref5, out) <= BERR
+    assert names == {"hrpb_quad_f32", "hrpb_brick_f32_rolling"}
+    with pytest.raises(cs.CuteError):
+        cs.SPMM_TC(h5, 128, operand_residency=3)
 
 
 def test_csr_comparison_kernels(cs, orc, torch_cuda):
