@@ -573,7 +573,8 @@ class SPMM_TC:
         _check(load_library().cute_spmm_plan_info(self._plan, C.byref(info)), "cute_spmm_plan_info")
         self.info = {k: getattr(info, k) for k, _ in cute_plan_info._fields_ if k != "reserved"}
         self.numRowPanelsSplit = info.numChunks
-        self.kernel_name = (("hrpb_quad_rows_f32" if info.fusedLaunch else "hrpb_quad_f32") if info.mfmaShape == 2 else
+        self.kernel_name = ("csr_rows_batched" if info.numChunks == 0 else
+                            ("hrpb_quad_rows_f32" if info.fusedLaunch else "hrpb_quad_f32") if info.mfmaShape == 2 else
                             "hrpb_brick_rows_f32" if info.fusedLaunch else
                             "hrpb_brick_bf16x3" if info.precision == PREC_BF16X3 else
                             "hrpb_brick_f32_rolling" if info.pipeline == 1 else "hrpb_brick_f32")

@@ -676,17 +676,30 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     }
     if (t.chunk_order > 3) { delete p; return CUTE_ERR_ARG; }
     p->info.dealtChunks = 0;
-    // A launch larger than the device starts its work-groups in list order as slots come free.  If its items differ
-    // widely in length (the longest at least four times the mean), the long ones go first, so that they run from the
-    // start and the short ones fill the gaps they leave; items are ordered by the power of two of their length only,
-    // so neighbours of similar length stay neighbours and keep sharing B rows in the L2.
+    // A launch larger than the device starts its work-groups in list order as slots come free, and every XCD walks
+    // its own eighth of the list.  In panel order that goes wrong in two ways: long items that start late keep the
+    // launch waiting, and a matrix whose heavy panels sit together (the hub vertices of an R-MAT graph are its first
+    // rows) gives one XCD most of the work.  So if the items differ widely in length (the longest at least four times
+    // the mean), or the eighths of the list differ by more than a tenth in work, the long items go first and the list
+    // is dealt round-robin to the XCDs: items are ordered by the power of two of their length only, so neighbours of
+    // similar length stay neighbours and keep sharing B rows in the L2.
     bool longest_first = t.chunk_order == 3;
     if (t.chunk_order == 0 && !chunks.empty()) {
         const uint64_t resident = uint64_t(c.num_cus) * 4u * ((p->shape == 2 || p->ng == 1) ? 8u : 4u);
         uint64_t total = 0;
         uint32_t longest = 0;
         for (const uint4 &ck : chunks) { total += ck.y - ck.x; longest = std::max(longest, ck.y - ck.x); }
-        longest_first = uint64_t(chunks.size()) * num_slabs > resident && uint64_t(longest) * chunks.size() >= 4u * total;
+        const uint32_t groups = (uint32_t(chunks.size()) + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
+        const size_t span = size_t((groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd) * cute_dev::kWavesPerGroup;
+        uint64_t fullest = 0;
+        for (uint32_t x = 0; x < cute_dev::kNumXcd; ++x) {
+            uint64_t work = 0;
+            for (size_t i = std::min(chunks.size(), x * span); i < std::min(chunks.size(), (x + 1) * span); ++i) work += chunks[i].y - chunks[i].x + 2u;
+            fullest = std::max(fullest, work);
+        }
+        const uint64_t even = (total + 2u * chunks.size() + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
+        longest_first = uint64_t(chunks.size()) * num_slabs > resident &&
+                        (uint64_t(longest) * chunks.size() >= 4u * total || fullest * 10u > even * 11u);
     }
     if (longest_first && !chunks.empty()) {
         std::vector<uint4> sorted(chunks);
