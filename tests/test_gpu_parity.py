@@ -391,6 +391,44 @@ def test_work_items_dealt_by_length(cs, orc, torch_cuda):
         cs.SPMM_TC(h5, 128, operand_residency=3)
 
 
+def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
+    """An upload sends the CSR arrays and the one MFMA layout the planner's default rules would use (none when every
+    panel would go to the row kernel); a plan that asks for the other one builds it then, from the device copy of the
+    CSR arrays -- also after the host arrays the format was made from have been overwritten."""
+    rng = np.random.default_rng(12)
+    A = cs.gen_config(2, 1 / 16.0)                                  # stencil: the default rules pick the quad lists
+    rp, cl, vl = A.rowPtr.copy(), A.cols.copy(), A.vals.copy()
+    h = cs.HRPB(A.M, A.K, rp, cl, vl)
+    B = rng.standard_normal((A.K, 64)).astype(np.float32)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+    csr_bytes = (A.M + 1) * 4 + A.nnz * 8
+    h.upload()
+    after_upload = h.device_bytes()
+    assert after_upload > csr_bytes
+    out, plan = _run(cs, torch_cuda, h, B)
+    assert plan.info["mfmaShape"] == 2 and h.device_bytes() == after_upload           # nothing more was needed
+    h.cols[:] = 0                                                                      # the borrowed host arrays go away
+    h.vals[:] = 0
+    out2, plan2 = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=1)
+    assert h.device_bytes() > after_upload                                             # the brick tiles were built now
+    for o in (out, out2):
+        assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, o) <= BERR
+    grown = h.device_bytes()
+    _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=1, pipeline=2)
+    assert h.device_bytes() == grown                                                   # built once
+    # every panel to the row kernel: the upload holds the CSR arrays only, until a plan forces an MFMA kernel
+    U = cs.gen_config(1)
+    hu = cs.HRPB(U.M, U.K, U.rowPtr, U.cols, U.vals)
+    hu.upload()
+    assert hu.device_bytes() == (U.M + 1) * 4 + U.nnz * 8
+    Bu = rng.standard_normal((U.K, 32)).astype(np.float32)
+    refu = orc.spmm_csr(U.rowPtr, U.cols, U.vals, Bu)
+    for kw in (dict(), dict(path=cs.PATH_BRICK, mfma_shape=2), dict(path=cs.PATH_BRICK, mfma_shape=1)):
+        out, _ = _run(cs, torch_cuda, hu, Bu, **kw)
+        assert cs.backward_error(U.rowPtr, U.cols, U.vals, Bu, refu, out) <= BERR, kw
+    assert hu.device_bytes() > (U.M + 1) * 4 + U.nnz * 8
+
+
 def test_csr_comparison_kernels(cs, orc, torch_cuda):
     torch = torch_cuda
     A = cs.gen_config(2, 1 / 16.0)
