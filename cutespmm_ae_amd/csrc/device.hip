@@ -281,6 +281,11 @@ int build_bricks(cute_hrpb_dev *d, const cute_hrpb_host *h)
     if (rc == CUTE_OK) {
         d->bytes += uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + (t.numVals + 64) * 4;
         d->haveBricks = true;
+    } else {                                  // nothing half-built stays behind: a later plan may try again
+        (void)hipFree(d->dHdr);
+        (void)hipFree(d->dVals);
+        d->dHdr = nullptr;
+        d->dVals = nullptr;
     }
     cute_hrpb_tiled_release(&t);
     return rc;
@@ -297,6 +302,11 @@ int build_quads(cute_hrpb_dev *d, const uint32_t *rowPtr, const uint32_t *cols, 
     if (rc == CUTE_OK) {
         d->bytes += d->qrecsHost.size() * 4 + packed.size() * 4;
         d->haveQuads = true;
+    } else {
+        (void)hipFree(d->dQRecs);
+        (void)hipFree(d->dQVals);
+        d->dQRecs = nullptr;
+        d->dQVals = nullptr;
     }
     return rc;
 }
@@ -900,8 +910,9 @@ int time_launches(hipStream_t s, int warmup, int iters, float *ms_out, Launch la
 {
     if (iters < 1 || !ms_out) return CUTE_ERR_ARG;
     std::vector<hipEvent_t> ev(size_t(iters) * 2, nullptr);
-    for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
     int rc = CUTE_OK;
+    for (auto &e : ev)
+        if (rc == CUTE_OK && hipEventCreate(&e) != hipSuccess) rc = CUTE_ERR_HIP;
     for (int i = 0; i < warmup && rc == CUTE_OK; ++i) rc = launch();
     for (int i = 0; i < iters && rc == CUTE_OK; ++i) {
         (void)hipEventRecord(ev[2 * i], s);
@@ -911,7 +922,8 @@ int time_launches(hipStream_t s, int warmup, int iters, float *ms_out, Launch la
     if (rc == CUTE_OK && hipStreamSynchronize(s) != hipSuccess) rc = CUTE_ERR_HIP;
     for (int i = 0; i < iters && rc == CUTE_OK; ++i)
         if (hipEventElapsedTime(&ms_out[i], ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = CUTE_ERR_HIP;
-    for (auto &e : ev) (void)hipEventDestroy(e);
+    for (auto &e : ev)
+        if (e) (void)hipEventDestroy(e);
     return rc;
 }
 }  // namespace
@@ -977,10 +989,6 @@ bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, floa
     return true;
 }
 }  // namespace
-
-extern "C" {
-
-}  // extern "C"
 
 namespace {
 // The launches of one product; `partials` is where the pieces of cut panels store their tiles.
@@ -1141,7 +1149,7 @@ int cute_blocked_ell_spmm(const cute_blocked_ell_dev *d, const float *dB, float 
 float cute_gpu_csr_spmm(const uint32_t *rowPtr, const uint32_t *cols, const float *vals, uint32_t nnz, const float *hB,
                         float *hC, uint32_t m, uint32_t k, uint32_t n, int iters, int alg)
 {
-    if (!rowPtr || !hB || !hC || iters < 1) return -float(-CUTE_ERR_ARG);
+    if (!rowPtr || !hB || !hC || iters < 1) return float(CUTE_ERR_ARG);
     const DeviceContext &c = context();
     if (c.status != CUTE_OK) return float(c.status);
     uint32_t *dR = nullptr, *dCl = nullptr;

@@ -1,12 +1,21 @@
 // gfx950 device kernels of libcutespmm.
 //
-//   hrpb_brick_f32   one wavefront per (row-panel chunk, N slab); every non-empty 16x4
-//                    brick is one v_mfma_f32_16x16x4_f32 A operand taken straight from the
-//                    lane-order bitmap; B rows are gathered in the MFMA B-operand layout
-//                    (16 lanes read one contiguous row segment) so no LDS transpose is needed.
-//   csr_rows         one lane group per CSR row, lanes span N, (col, val) pairs broadcast
-//                    by lane shuffles; used for sparse panels and as a plain CSR kernel.
-//   csr_thread_per_element / csr_wave_scalar   the simple CSR comparison kernels.
+//   hrpb_brick_f32_rolling   one wavefront per (row-panel chunk, N slab) over the brick tiles; every non-empty
+//                    16x4 brick is one v_mfma_f32_16x16x4_f32 A operand taken straight from the lane-order
+//                    bitmap; B rows are gathered in the MFMA B-operand layout (16 lanes read one contiguous
+//                    row segment), so no LDS transpose is needed.  One operand set, refilled behind the MFMAs.
+//   hrpb_brick_f32   the same work with two whole operand sets in flight and 64-bit addressing (operands
+//                    beyond the 32-bit offsets of the rolling variant).
+//   hrpb_brick_bf16x3   the brick tiles on the bf16 matrix pipeline: operands split into bf16 high and low
+//                    parts in registers, three v_mfma_f32_16x16x16_bf16 per block and 16 columns.
+//   hrpb_quad_f32    quad lists: v_mfma_f32_4x4x1_16B_f32 over 16 (row group, column) pairs at a time, so
+//                    only occupied 4-row column pieces cost matrix time.
+//   csr_rows_batched one lane group per CSR row, lanes span N, 8 (col, val) pairs in flight; the kernel
+//                    for panels with too little reuse for the matrix cores.
+//   hrpb_quad_rows_f32 / hrpb_brick_rows_f32   MFMA work items and sparse rows of a mixed plan in one launch.
+//   reduce_partials  adds up the partial tiles of panels that were cut, in chunk order (no atomics).
+//   blocked_ell_f32  fp32 MFMA over the dense blocks of a Blocked-ELL matrix.
+//   csr_rows / csr_thread_per_element / csr_wave_scalar   the simple CSR comparison kernels.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

@@ -358,7 +358,9 @@ typedef enum cute_precision {
     CUTE_PREC_BF16X3 = 1       /* brick kernel on the bf16 matrix pipeline: operands split into bf16 hi + lo in registers,
                                   three products per block, fp32 accumulation; error below 2^-16 per product.  Used where it
                                   exists (brick tiles, N a multiple of 4, 32-bit offsets), fp32 elsewhere: cute_plan_info.precision
-                                  says which.  Panels the planner sends to the row kernel are always fp32. */
+                                  says which.  Panels the planner sends to the row kernel are always fp32.  Operands must
+                                  stay inside bf16's range: a magnitude above about 3.39e38 rounds to infinity in the split, and
+                                  low parts below about 1e-38 are flushed (such values keep 8 bits instead of 16). */
 } cute_precision;
 
 typedef struct cute_tunables {
