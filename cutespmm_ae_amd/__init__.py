@@ -27,6 +27,7 @@ ABI_SYMBOLS = [
     "cute_gen_matrix", "cute_gen_dense",
     "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
     "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run", "cute_spmm_run_static",
+    "cute_spmm_run_scratch", "cute_spmm_plan_scratch_bytes", "cute_device_layout",
     "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
     "cute_device_info",
     "cute_coo_read", "cute_coo_save_mtx", "cute_coo_release", "cute_coo_to_csr", "cute_csr_i32_release",
@@ -189,6 +190,10 @@ def load_library():
     lib.cute_spmm_plan_free.argtypes = [C.c_void_p]
     lib.cute_spmm_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.cute_spmm_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.cute_spmm_run_scratch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]
+    lib.cute_spmm_plan_scratch_bytes.restype = C.c_uint64
+    lib.cute_spmm_plan_scratch_bytes.argtypes = [C.c_void_p]
+    lib.cute_device_layout.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_uint64), C.POINTER(C.c_int)]
     lib.cute_csr_spmm_dev.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_uint32, C.c_uint32, C.c_void_p]
     lib.cute_gpu_csr_spmm.restype = C.c_float
@@ -596,6 +601,21 @@ class SPMM_TC:
                "cute_spmm_run_static")
         return MatC
 
+    @property
+    def scratch_bytes(self):
+        """Bytes of partial tiles one launch stores (0 when no panel is cut)."""
+        return int(load_library().cute_spmm_plan_scratch_bytes(self._plan))
+
+    def run_scratch(self, MatB, MatC, scratch, stream=None):
+        """``run`` with the partial tiles in ``scratch`` (a GPU tensor of at least ``scratch_bytes`` bytes, or None
+        when that is 0): one plan can then run on several streams at once, each call with its own buffer."""
+        self._check_shapes(MatB, MatC)
+        ptr = C.c_void_p(scratch.data_ptr()) if scratch is not None else C.c_void_p()
+        nbytes = scratch.numel() * scratch.element_size() if scratch is not None else 0
+        _check(load_library().cute_spmm_run_scratch(self._plan, _dev_ptr(MatB), _dev_ptr(MatC), _stream_ptr(stream), ptr, nbytes),
+               "cute_spmm_run_scratch")
+        return MatC
+
     def time(self, MatB, MatC, warmup=3, iters=20, stream=None):
         """Per-launch milliseconds (HIP events on the launch stream)."""
         self._check_shapes(MatB, MatC)
@@ -691,7 +711,10 @@ def device_info():
     cus, ws = C.c_int(), C.c_int()
     name = C.create_string_buffer(64)
     _check(load_library().cute_device_info(C.byref(cus), C.byref(ws), name, 64), "cute_device_info")
-    return dict(num_cus=cus.value, wave_size=ws.value, arch=name.value.decode())
+    xcds, per, whole, cache = C.c_int(), C.c_int(), C.c_int(), C.c_uint64()
+    _check(load_library().cute_device_layout(C.byref(xcds), C.byref(per), C.byref(cache), C.byref(whole)), "cute_device_layout")
+    return dict(num_cus=cus.value, wave_size=ws.value, arch=name.value.decode(), num_xcds=xcds.value, cus_per_xcd=per.value,
+                cache_bytes=cache.value, whole_chip=bool(whole.value))
 
 
 # --------------------------------------------------------------------------------------

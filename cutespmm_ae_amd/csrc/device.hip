@@ -25,8 +25,37 @@ constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels n
 // stays below the time the operands take to stream at 4 TB/s; on R-MAT graphs, where it is 1.4 to 1.7 times
 // that, the two kernels are within 10 % of each other either way and the rule above keeps deciding.  While the
 // operands fit the cache the quad kernel is level or ahead.
-constexpr uint64_t kInfinityCacheBytes = 256ull << 20;
 constexpr double kStreamBytesPerSecond = 4.0e12, kSimdCyclesPerSecond = 1024 * 2.4e9, kCyclesPerBrickTile = 32.0;
+
+// Which MFMA kernel serves the panels that go to the matrix cores (1 brick tiles, 2 quad lists).
+//   slots   list slots of the quad lists (pairs plus padding): the quad kernel pays 8 matrix cycles and one
+//           256-byte piece of a B row per slot and 64 columns
+//   bricks  16x4 bricks: the brick kernel pays 32 matrix cycles per brick and 16 columns, however empty the brick
+//   blocks  16-column blocks: the brick kernel requests 16 row pieces per block (padding columns included)
+// A launch fed from a cache is bound by what it issues, and the two kernels cross at about 8 slots per brick
+// (measured on the benchmark matrices and on the reference's 43).  A launch fed from HBM is bound by the
+// memory system, and what counts there is how many row pieces a kernel requests and how wide they are: the
+// brick kernel asks for a B row once per panel, in pieces of 512 contiguous bytes from N = 128 on; the quad
+// kernel once per 4-row group that uses it, in 256-byte pieces that two wavefronts request at different
+// times.  Measured with operands no cache holds: 9-point stencils (1.25 slots per brick-kernel fetch) run
+// 7-25 % faster through the brick kernel at 16 384 to 262 144 rows and N = 64..512, 5-point stencils (1.0)
+// 5-8 % slower; from a cache the quad kernel is level or up to 20 % ahead on both.  So unless the caller
+// says that the operands stay cache-resident (operand_residency = 2, a tight loop over the same buffers that
+// fit the Infinity Cache), a matrix whose quad lists need more than 1.1 fetches per brick-kernel fetch goes to
+// the brick kernel -- as long as its matrix work stays below the time the operands take to stream at 4 TB/s
+// (on R-MAT graphs it is 1.4-1.7 times that, and the quad kernel keeps them).
+int choose_mfma_shape(uint64_t slots, uint64_t bricks, uint64_t blocks, uint64_t rows_and_cols, uint64_t nnz, uint32_t N,
+                      uint32_t residency, uint64_t cache_bytes)
+{
+    int shape = slots < kSlotsPerBrick * bricks ? 2 : 1;
+    const bool resident = residency == 2 && rows_and_cols * N * sizeof(float) <= cache_bytes;
+    if (shape == 2 && !resident && slots * 10u > blocks * 16u * 11u) {
+        const double matrix_s = double(bricks) * double((N + 15u) / 16u) * kCyclesPerBrickTile / kSimdCyclesPerSecond;
+        const double stream_s = (double(rows_and_cols) * N * 4.0 + double(nnz) * 8.0) / kStreamBytesPerSecond;
+        if (matrix_s <= stream_s) shape = 1;
+    }
+    return shape;
+}
 
 inline int hip_fail(hipError_t e, const char *what, int line)
 {
@@ -44,6 +73,15 @@ struct DeviceContext {
     int device = 0;
     int num_cus = 0;
     int wave_size = 0;
+    // What the planner assumes about the part of the chip this device is.  A whole MI355X (SPX mode) shows 256
+    // compute units in 8 XCDs of 32, each XCD with its own 4 MiB L2, and 256 MiB of Infinity Cache; in the
+    // partitioned modes a device is 4, 2 or 1 of those XCDs with its share of the cache.  The kernels' mapping of
+    // work-groups to contiguous panel ranges is written for 8 XCDs and stays a valid, locality-preserving order
+    // on fewer (a device with x XCDs walks 8/x ranges per XCD); the model of where wavefronts land, which only
+    // orders work items, is used on the whole chip alone.
+    int num_xcds = 8;
+    bool whole_chip = false;
+    uint64_t cache_bytes = 256ull << 20;
     std::string arch;
 };
 
@@ -69,6 +107,9 @@ const DeviceContext &context()
             g_hip_error = "device is " + c.arch + ", this library is built for gfx950 only";
             return c;
         }
+        if (c.num_cus > 0 && c.num_cus % 32 == 0 && c.num_cus / 32 <= 8) c.num_xcds = c.num_cus / 32;
+        c.whole_chip = c.num_cus == 256;
+        c.cache_bytes = (256ull << 20) * uint64_t(c.num_xcds) / 8u;
         c.status = CUTE_OK;
         return c;
     }();
@@ -155,6 +196,7 @@ struct cute_spmm_plan {
     uint32_t unitRows = CUTE_TM;        // rows of one panel / strip / piece
     float *dPartials = nullptr;         // pieces x unitRows rows of N floats; owned by the plan, so a plan runs on one stream at a time
     uint64_t partialBytes = 0;
+    void *staticScratch = nullptr;      // device address of the library's static scratch array on the plan's device
     uint32_t *dRowList = nullptr;
     uint32_t numRows = 0;
     cute_dev::XcdRanges rowRanges{};   // row-kernel blocks of each XCD, balanced by nonzeros
@@ -244,6 +286,17 @@ int cute_device_info(int *num_cus, int *wave_size, char *arch_name, size_t arch_
     return CUTE_OK;
 }
 
+int cute_device_layout(int *num_xcds, int *cus_per_xcd, uint64_t *cache_bytes, int *whole_chip)
+{
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    if (num_xcds) *num_xcds = c.num_xcds;
+    if (cus_per_xcd) *cus_per_xcd = c.num_cus / c.num_xcds;
+    if (cache_bytes) *cache_bytes = c.cache_bytes;
+    if (whole_chip) *whole_chip = c.whole_chip ? 1 : 0;
+    return CUTE_OK;
+}
+
 void cute_hrpb_dev_free(cute_hrpb_dev *d)
 {
     if (!d) return;
@@ -271,6 +324,9 @@ int build_bricks(cute_hrpb_dev *d, const cute_hrpb_host *h)
     cute_hrpb_tiled t;
     int rc = cute_hrpb_retile(h, &t);
     if (rc != CUTE_OK) return rc;
+    // the kernels take numVals as the position of the zero pad behind the values: the tiles must hold
+    // exactly one value per entry of the matrix, or masked lanes would read real values
+    if (t.numVals != d->numVals) { cute_hrpb_tiled_release(&t); return CUTE_ERR_FORMAT; }
     rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
     if (rc == CUTE_OK) {
         // one wavefront of zero padding behind the values: a lane without a nonzero reads its operand there
@@ -408,7 +464,7 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
     if (rc == CUTE_OK) {
         // Which MFMA layout would the planner's default rules use (see cute_spmm_plan_create)?  Build that one now.
         const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
-        uint64_t slots = 0, bricks = 0;
+        uint64_t slots = 0, bricks = 0, blocks = 0;
         for (uint32_t q = 0; q < d->P; ++q) {
             if (d->brp[q + 1] == d->brp[q]) continue;
             const uint32_t list_slots = (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
@@ -416,12 +472,12 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
             if (float(d->panelNnz[q]) < kMinReuse * float(fetches) && d->panelMaxRow[q] <= kMaxRowForRows) continue;   // row kernel
             slots += list_slots;
             bricks += (d->panelCols[q] + 3u) / 4u;
+            blocks += d->brp[q + 1] - d->brp[q];
         }
-        // (the width is not known yet: 128 columns stand in for it in the rule for operands beyond the cache)
-        const bool beyond_cache = (uint64_t(d->K) + d->M) * 128u * sizeof(float) > kInfinityCacheBytes &&
-                                  double(bricks) * 8.0 * kCyclesPerBrickTile / kSimdCyclesPerSecond <=
-                                      (double(uint64_t(d->K) + d->M) * 512.0 + double(d->nnz) * 8.0) / kStreamBytesPerSecond;
-        if (bricks) rc = (slots < kSlotsPerBrick * bricks && !beyond_cache) ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
+        // (the width is not known yet: 128 columns stand in for it)
+        if (bricks)
+            rc = choose_mfma_shape(slots, bricks, blocks, uint64_t(d->K) + d->M, d->nnz, 128u, 0u, c.cache_bytes) == 2
+                     ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
     }
     if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
     *out = d;
@@ -524,7 +580,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     // (not when B and C come from HBM: there the wider row pieces of two column groups count for more)
     if (t.operand_residency > 2) { delete p; return CUTE_ERR_ARG; }
     const bool beyond_cache = t.operand_residency ? t.operand_residency == 1
-                                                  : (uint64_t(d->K) + d->M) * N * sizeof(float) > kInfinityCacheBytes;
+                                                  : (uint64_t(d->K) + d->M) * N * sizeof(float) > c.cache_bytes;
     if (p->ng == 2 && t.brick_groups == 0 && n_brick && n_rows && !beyond_cache) {
         const uint64_t row_blocks = (uint64_t(n_rows) * CUTE_TM * p->rows_slabs + (256u >> p->rows_logl) - 1) / (256u >> p->rows_logl);
         const uint64_t groups = (uint64_t(n_brick) * ((N + 127u) / 128u) + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
@@ -545,18 +601,14 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         // instead of once per panel, and pad their lists.  Measured break-even on the benchmark
         // matrices and on the reference's 43: about 8 list slots (pairs plus padding) per brick.
         const uint32_t lists = d->quadRows == 4 ? 4u : 1u;     // list units per panel
-        uint64_t slots = 0, bricks = 0;
+        uint64_t slots = 0, bricks = 0, blocks = 0;
         for (uint32_t q = 0; q < d->P; ++q)
             if (!to_rows[q]) {
                 slots += uint64_t(d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
                 bricks += (d->panelCols[q] + 3u) / 4u;
+                blocks += d->brp[q + 1] - d->brp[q];
             }
-        p->shape = slots < kSlotsPerBrick * bricks ? 2 : 1;
-        if (beyond_cache) {
-            const double matrix_s = double(bricks) * double((N + 15u) / 16u) * kCyclesPerBrickTile / kSimdCyclesPerSecond;
-            const double stream_s = (double(uint64_t(d->K) + d->M) * N * 4.0 + double(d->nnz) * 8.0) / kStreamBytesPerSecond;
-            if (matrix_s <= stream_s) p->shape = 1;
-        }
+        p->shape = choose_mfma_shape(slots, bricks, blocks, uint64_t(d->K) + d->M, d->nnz, N, t.operand_residency, c.cache_bytes);
     }
     if (p->shape == 2 && !(offsets_fit && (d->numQuadVals + 64u) * 4u <= 0xffffffffull)) p->shape = 1;
     // bf16x3 exists for the rolling brick kernel with four columns per lane; any other shape computes in fp32
@@ -741,7 +793,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
         }
         p->info.dealtChunks = 2;
     } else
-    if (t.chunk_order != 1 && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
+    if (t.chunk_order != 1 && c.whole_chip && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
         p->info.dealtChunks = deal_chunks(chunks, num_slabs, uint32_t(c.num_cus) / cute_dev::kNumXcd,
                                           p->shape == 2 || p->ng == 1 ? 8u : 4u, t.chunk_order == 2) ? 1u : 0u;
     // the layout this plan's MFMA kernel reads, if the upload has not built it
@@ -774,8 +826,7 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (rc == CUTE_OK) {
         // cute_spmm_run_static's scratch: its address on this device is looked up here, at set-up, so that the
         // run call itself is nothing but kernel launches
-        void *unused = nullptr;
-        rc = static_scratch(&unused);
+        rc = static_scratch(&p->staticScratch);
     }
     if (rc != CUTE_OK) { cute_spmm_plan_free(p); return rc; }
     p->numFixups = uint32_t(fixups.size());
@@ -1080,10 +1131,25 @@ int cute_spmm_run_static(cute_spmm_plan *p, const float *dB, float *dC, void *st
                       std::to_string(uint64_t(CUTE_STATIC_SCRATCH_BYTES));
         return CUTE_ERR_SCRATCH;
     }
-    void *ptr = nullptr;
-    const int rc = static_scratch(&ptr);      // a table look-up: the address was fetched when the plan was made
-    if (rc != CUTE_OK) return rc;
-    return run_with(p, dB, dC, stream, static_cast<float *>(ptr));
+    return run_with(p, dB, dC, stream, static_cast<float *>(p->staticScratch));   // the address was fetched when the plan was made
+}
+
+uint64_t cute_spmm_plan_scratch_bytes(const cute_spmm_plan *p) { return p ? p->partialBytes : 0; }
+
+// The same launches with the partial tiles in memory the caller brings: one plan can then run on several
+// streams at once, each call with a buffer of its own.
+int cute_spmm_run_scratch(cute_spmm_plan *p, const float *dB, float *dC, void *stream, void *scratch, uint64_t scratch_bytes)
+{
+    if (!p) return CUTE_ERR_ARG;
+    if (p->partialBytes) {
+        if (!scratch || (reinterpret_cast<uintptr_t>(scratch) & 15u)) return CUTE_ERR_ARG;
+        if (scratch_bytes < p->partialBytes) {
+            g_hip_error = "plan needs " + std::to_string(p->partialBytes) + " bytes of partial tiles, the caller's scratch holds " +
+                          std::to_string(scratch_bytes);
+            return CUTE_ERR_SCRATCH;
+        }
+    }
+    return run_with(p, dB, dC, stream, static_cast<float *>(scratch));
 }
 
 int cute_csr_spmm_dev(int alg, const uint32_t *dRowPtr, const uint32_t *dCols, const float *dVals, const float *dB,

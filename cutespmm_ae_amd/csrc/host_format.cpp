@@ -101,6 +101,10 @@ struct Triplet { uint32_t r, c; float v; };
 // come out in file order, a mirrored entry right behind its original, exactly where the
 // reference's loader puts them (IO.cu:71-84).  A file without a banner is read the way the
 // reference reads every file: "symmetric" anywhere on the first line means mirror.
+// Largest dimension a size line may state: the reference parses it with stoi (IO.cu:23-29), which throws
+// beyond INT_MAX -- and a forged line must not turn into a multi-gigabyte row-pointer allocation.
+constexpr long long kMaxFileDim = 0x7FFFFFFFll - 16;
+
 int read_triplets(const char *begin, const char *end_, long long &m, long long &k, std::vector<Triplet> &out)
 {
     LineCursor lc{begin, end_};
@@ -126,8 +130,11 @@ int read_triplets(const char *begin, const char *end_, long long &m, long long &
     if (!have_size) return CUTE_ERR_IO;
     const char *s = b;
     if (next_int(s, e, m) != 1 || next_int(s, e, k) != 1 || m <= 0 || k <= 0) return CUTE_ERR_IO;
-    if (m > 0xFFFFFFF0ll || k > 0xFFFFFFF0ll) return CUTE_ERR_SHAPE;
+    if (m > kMaxFileDim || k > kMaxFileDim) return CUTE_ERR_SHAPE;
     if (mirror && bn.present && m != k) return CUTE_ERR_FORMAT;
+    // a coordinate file announces its number of entries; what follows must be exactly that many
+    long long announced = -1, seen = 0;
+    if (!bn.array && (next_int(s, e, announced) != 1 || announced < 0)) return CUTE_ERR_FORMAT;
     auto push = [&](long long r, long long c, float v) {
         out.push_back(Triplet{uint32_t(r - 1), uint32_t(c - 1), v});
         if (mirror && r != c) out.push_back(Triplet{uint32_t(c - 1), uint32_t(r - 1), mirror_sign * v});
@@ -165,8 +172,9 @@ int read_triplets(const char *begin, const char *end_, long long &m, long long &
             if (endp != w) v = static_cast<float>(d);
         }
         push(r, c, v);
+        ++seen;
     }
-    return CUTE_OK;
+    return seen == announced ? CUTE_OK : CUTE_ERR_FORMAT;
 }
 
 int csr_from_triplets(long long m, long long k, const std::vector<Triplet> &t, cute_csr *out)
@@ -232,7 +240,7 @@ extern "C" int cute_mtx_read(const char *path, int keep_values, cute_csr *out)
     long long m = 0, k = 0;
     const char *s = b;
     if (next_int(s, e, m) != 1 || next_int(s, e, k) != 1 || m <= 0 || k <= 0) return CUTE_ERR_IO;
-    if (m > 0xFFFFFFF0ll || k > 0xFFFFFFF0ll) return CUTE_ERR_SHAPE;
+    if (m > kMaxFileDim || k > kMaxFileDim) return CUTE_ERR_SHAPE;   // where the reference's stoi throws
     const uint32_t M = uint32_t((m - 1) / CUTE_TM + 1) * CUTE_TM;   // IO.cu:30
     const uint32_t K = uint32_t((k - 1) / CUTE_TK + 1) * CUTE_TK;   // IO.cu:31
     const char *data_begin = lc.p;

@@ -115,13 +115,21 @@ int cute_coo_read(const char *path, cute_coo *out)
         char *p = const_cast<char *>(b), *q;
         dy = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; p = q;
         dx = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; p = q;
-        if (!bn.array) { hdr = std::strtoll(p, &q, 10); if (q == p) return CUTE_ERR_IO; }
+        if (!bn.array) {
+            // (the count must stand on the size line itself: strtoll would walk on into the next line)
+            while (p < e && (*p == ' ' || *p == '\t' || *p == '\r')) ++p;
+            if (p >= e) return CUTE_ERR_FORMAT;
+            hdr = std::strtoll(p, &q, 10);
+            if (q == p) return CUTE_ERR_IO;
+        }
     }
-    if (dy <= 0 || dx <= 0 || dy > 0x7FFFFFFF || dx > 0x7FFFFFFF || hdr < 0) return CUTE_ERR_SHAPE;
+    if (dy <= 0 || dx <= 0 || dy > 0x7FFFFFFF || dx > 0x7FFFFFFF || hdr < 0 || hdr > 0x7FFFFFFF) return CUTE_ERR_SHAPE;
     if (bn.present && symmetric && dy != dx) return CUTE_ERR_FORMAT;
     struct Pt { int r, c; float v; };
     std::vector<Pt> pts;
-    pts.reserve(size_t(hdr) * (symmetric ? 2 : 1));
+    // (an entry takes at least four bytes of the file: a forged count must not size the allocation)
+    pts.reserve(std::min<size_t>(size_t(hdr), buf.size() / 4) * (symmetric ? 2 : 1));
+    long long seen = 0;
     if (bn.array) {
         // column-major, one value per line; symmetric: lower triangle with, skew-symmetric without the diagonal
         long long r = bn.symmetry == 2 ? 2 : 1, c = 1;
@@ -164,7 +172,11 @@ int cute_coo_read(const char *path, cute_coo *out)
             if (y > dy || x > dx) return CUTE_ERR_RANGE;
             pts.push_back(Pt{int(y - 1), int(x - 1), mirror_sign * float(v)});
         }
+        ++seen;
     }
+    // SparseCoo.hpp:128-149 reads every line but takes nnz from the size line, so a file whose entries do
+    // not match its own size line leaves it with arrays and a count that disagree; such a file is refused here
+    if (!bn.array && seen != hdr) return CUTE_ERR_FORMAT;
     if (pts.size() > 0x7FFFFFFFull) return CUTE_ERR_SHAPE;
     std::stable_sort(pts.begin(), pts.end(), [](const Pt &a, const Pt &b2) {           // :152
         return a.r != b2.r ? a.r < b2.r : a.c < b2.c;

@@ -376,9 +376,11 @@ typedef struct cute_tunables {
     uint32_t chunk_order;      /* MFMA work items: 0 library's choice (a launch that is resident at once: dealt to the SIMDs longest
                                   first where that shortens the fullest SIMD; a larger launch whose longest item is four times the
                                   mean: long items first); 1 always in panel order; 2 always dealt; 3 always long items first */
-    uint32_t operand_residency; /* where B and C are when a launch starts: 0 decided by size (from HBM when they exceed the 256 MiB
-                                  Infinity Cache together), 1 from HBM (a product on data no cache holds), 2 cache-resident
-                                  (the same operands again and again).  Chooses between the MFMA kernels, nothing else. */
+    uint32_t operand_residency; /* where B and C are when a launch starts: 0 unknown -- planned like 1, because a product on
+                                  fresh data finds its operands in HBM whatever their size; 1 from HBM (a product on data no
+                                  cache holds); 2 cache-resident (a tight loop over the same operands that fit the 256 MiB
+                                  Infinity Cache together; ignored when they do not).  Chooses between the MFMA kernels
+                                  (and, for 1, keeps two column groups per lane in mixed plans), nothing else. */
     uint32_t reserved[1];
 } cute_tunables;
 
@@ -432,6 +434,16 @@ int cute_spmm_run(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
 #define CUTE_STATIC_SCRATCH_BYTES (32u << 20)
 int cute_spmm_run_static(cute_spmm_plan *p, const float *dB, float *dC, void *stream);
 
+/* cute_spmm_run with the partial tiles of cut panels in a buffer the caller brings (device memory, 16-byte
+ * aligned, at least cute_spmm_plan_scratch_bytes(p) bytes; ignored when that is 0), so that one plan can run on
+ * several streams at the same time, each call with a buffer of its own.  The reference's kernel adds the
+ * pieces of a split panel into C with atomicAdd (kernel.cu:258-271) and needs no such buffer, at the price of
+ * results that depend on the order of arrival.  Too small a buffer gives CUTE_ERR_SCRATCH.  Same bits in C as
+ * cute_spmm_run. */
+uint64_t cute_spmm_plan_scratch_bytes(const cute_spmm_plan *p);
+int cute_spmm_run_scratch(cute_spmm_plan *p, const float *dB, float *dC, void *stream, void *scratch,
+                          uint64_t scratch_bytes);
+
 /* ------------------------------------------------------------------------------------
  * device: plain CSR SpMM kernels -- the fp32 CSR comparison path.  Replaces
  * GPU_CSR_cuSPARSE_NEW (spmm.cu:860-960); the three algorithms restate the simple kernels
@@ -462,6 +474,11 @@ int cute_csr_spmm_time(int alg, const cute_hrpb_dev *d, const float *dB, float *
                        void *stream, int warmup, int iters, float *ms_out);
 
 int cute_device_info(int *num_cus, int *wave_size, char *arch_name, size_t arch_cap);
+/* What the planner assumes about the device: the number of XCDs it spans (8 for a whole MI355X, 256 compute units;
+ * 4, 2 or 1 in the partitioned modes), compute units per XCD, its share of the Infinity Cache, and whether it
+ * is the whole chip (the model of where wavefronts land, which orders work items, is used there only).  Stands
+ * where spmm.cu:290-690 tabulates resident warps, blocks and SM counts per machine. */
+int cute_device_layout(int *num_xcds, int *cus_per_xcd, uint64_t *cache_bytes, int *whole_chip);
 
 #ifdef __cplusplus
 }

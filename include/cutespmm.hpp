@@ -190,6 +190,13 @@ public:
             throw cute::Error(CUTE_ERR_ARG, "SPMM_TC::run: MatA, active_cols_vec, sizePtr are not this plan's HRPB device fields");
         run(MatB, MatC, nullptr);
     }
+    // With the partial tiles of cut panels in the caller's buffer (scratch_bytes() bytes of device memory):
+    // one plan can then run on several streams at once.
+    uint64_t scratch_bytes() const { return cute_spmm_plan_scratch_bytes(plan_); }
+    void run(const float *MatB, float *MatC, void *stream, void *scratch, uint64_t bytes)
+    {
+        cute::check(cute_spmm_run_scratch(plan_, MatB, MatC, stream, scratch, bytes), "SPMM_TC::run");
+    }
     cute_spmm_plan *plan() { return plan_; }
     ~SPMM_TC() { cute_spmm_plan_free(plan_); }
     SPMM_TC(const SPMM_TC &) = delete;

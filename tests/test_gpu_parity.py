@@ -381,14 +381,52 @@ def test_work_items_dealt_by_length(cs, orc, torch_cuda):
     h5 = cs.HRPB(A5.M, A5.K, A5.rowPtr, A5.cols, A5.vals)
     B5 = rng.standard_normal((A5.K, 128)).astype(np.float32)
     ref5 = orc.spmm_csr(A5.rowPtr, A5.cols, A5.vals, B5)
-    names = set()
-    for res in (0, 1, 2):
+    # (unknown is planned like "from HBM": a product on fresh data finds its operands there whatever their size)
+    for res, name in ((0, "hrpb_brick_f32_rolling"), (1, "hrpb_brick_f32_rolling"), (2, "hrpb_quad_f32")):
         out, plan = _run(cs, torch_cuda, h5, B5, operand_residency=res)
-        names.add(plan.kernel_name)
+        assert plan.kernel_name == name, (res, plan.kernel_name)
         assert cs.backward_error(A5.rowPtr, A5.cols, A5.vals, B5, ref5, out) <= BERR
-    assert names == {"hrpb_quad_f32", "hrpb_brick_f32_rolling"}
     with pytest.raises(cs.CuteError):
         cs.SPMM_TC(h5, 128, operand_residency=3)
+
+
+def _stencil5(g):
+    """5-point stencil on a g x g grid (rows padded to a multiple of 16), the shape of the reference's `obstclae`."""
+    idx = np.arange(g * g).reshape(g, g)
+    rows, cols = [], []
+    for di, dj in ((0, 0), (-1, 0), (1, 0), (0, -1), (0, 1)):
+        src = idx[max(0, -di):g - max(0, di), max(0, -dj):g - max(0, dj)]
+        dst = idx[max(0, di):g - max(0, -di), max(0, dj):g - max(0, -dj)]
+        rows.append(src.ravel())
+        cols.append(dst.ravel())
+    r, c = np.concatenate(rows), np.concatenate(cols)
+    o = np.lexsort((c, r))
+    r, c = r[o], c[o]
+    M = ((g * g + 15) // 16) * 16
+    rp = np.zeros(M + 1, np.int64)
+    np.add.at(rp, r + 1, 1)
+    vals = np.random.default_rng(g).uniform(-1, 1, len(c)).astype(np.float32)
+    return M, np.cumsum(rp).astype(np.uint32), c.astype(np.uint32), vals
+
+
+def test_default_kernel_choice(cs, orc, torch_cuda):
+    """The planner's default on the headline shape, pinned: the 65 536-row 9-point stencil at N = 128 goes to the
+    brick kernel unless the caller says that its operands stay cache-resident (its quad lists ask for 1.25 B-row
+    pieces per piece the brick kernel asks for); a 5-point stencil (1.0) stays on the quad kernel either way."""
+    A = cs.gen_config(2)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    assert cs.SPMM_TC(h, 128).kernel_name == "hrpb_brick_f32_rolling"
+    assert cs.SPMM_TC(h, 128, operand_residency=1).kernel_name == "hrpb_brick_f32_rolling"
+    assert cs.SPMM_TC(h, 128, operand_residency=2).kernel_name == "hrpb_quad_f32"
+    assert cs.SPMM_TC(h, 1024, operand_residency=2).kernel_name == "hrpb_brick_f32_rolling"   # 512 MiB: no cache holds that
+    M, rp, cl, vl = _stencil5(200)
+    h5 = cs.HRPB(M, M, rp, cl, vl)
+    B = np.random.default_rng(5).standard_normal((M, 128)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    for res in (0, 1, 2):
+        out, plan = _run(cs, torch_cuda, h5, B, operand_residency=res)
+        assert plan.info["mfmaShape"] == 2 and plan.kernel_name.startswith("hrpb_quad"), (res, plan.kernel_name)
+        assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
 
 
 def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
@@ -396,7 +434,7 @@ def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
     panel would go to the row kernel); a plan that asks for the other one builds it then, from the device copy of the
     CSR arrays -- also after the host arrays the format was made from have been overwritten."""
     rng = np.random.default_rng(12)
-    A = cs.gen_config(2, 1 / 16.0)                                  # stencil: the default rules pick the quad lists
+    A = cs.gen_config(2, 1 / 16.0)                                  # 9-point stencil: the default rules pick the brick tiles
     rp, cl, vl = A.rowPtr.copy(), A.cols.copy(), A.vals.copy()
     h = cs.HRPB(A.M, A.K, rp, cl, vl)
     B = rng.standard_normal((A.K, 64)).astype(np.float32)
@@ -406,15 +444,15 @@ def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
     after_upload = h.device_bytes()
     assert after_upload > csr_bytes
     out, plan = _run(cs, torch_cuda, h, B)
-    assert plan.info["mfmaShape"] == 2 and h.device_bytes() == after_upload           # nothing more was needed
+    assert plan.info["mfmaShape"] == 1 and h.device_bytes() == after_upload           # nothing more was needed
     h.cols[:] = 0                                                                      # the borrowed host arrays go away
     h.vals[:] = 0
-    out2, plan2 = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=1)
-    assert h.device_bytes() > after_upload                                             # the brick tiles were built now
+    out2, plan2 = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=2)
+    assert h.device_bytes() > after_upload                                             # the quad lists were built now
     for o in (out, out2):
         assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, o) <= BERR
     grown = h.device_bytes()
-    _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=1, pipeline=2)
+    _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK, mfma_shape=2, max_chunk_blocks=2)
     assert h.device_bytes() == grown                                                   # built once
     # every panel to the row kernel: the upload holds the CSR arrays only, until a plan forces an MFMA kernel
     U = cs.gen_config(1)

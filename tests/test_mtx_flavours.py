@@ -33,6 +33,9 @@ REFUSED = {
     "array_too_short": "%%MatrixMarket matrix array real general\n2 2\n1\n1\n1\n",
     "array_too_long": "%%MatrixMarket matrix array real general\n2 2\n1\n1\n1\n1\n1\n",
     "symmetric_not_square": "%%MatrixMarket matrix coordinate real symmetric\n2 3 1\n2 1 1.0\n",
+    "fewer_entries_than_announced": "%%MatrixMarket matrix coordinate real general\n3 3 3\n1 1 1.0\n",
+    "more_entries_than_announced": "%%MatrixMarket matrix coordinate real general\n3 3 1\n1 1 1.0\n2 2 1.0\n",
+    "no_entry_count": "%%MatrixMarket matrix coordinate real general\n3 3\n1 1 1.0\n",
 }
 
 
@@ -95,6 +98,27 @@ def test_refused_files(cs, tmp_path, name):
         with pytest.raises(cs.CuteError) as e:
             read()
         assert e.value.status == -9, name
+
+
+@pytest.mark.parametrize("dims", ["4000000000 4000000000 1", "2147483648 5 1", "5 2147483648 1"])
+def test_size_lines_beyond_int_are_refused(cs, tmp_path, dims):
+    """The reference parses the size line with stoi (IO.cu:23-29), which throws beyond INT_MAX; here every reader
+    returns a status instead of allocating row pointers for four billion rows."""
+    p = tmp_path / "huge.mtx"
+    p.write_text("%%MatrixMarket matrix coordinate real general\n" + dims + "\n1 1 1.0\n")
+    for read in (lambda: cs.MTX_READER(str(p)), lambda: cs.MTX_READER(str(p), keep_values=True), lambda: cs.SparseCoo(str(p))):
+        with pytest.raises(cs.CuteError) as e:
+            read()
+        assert e.value.status == -2, dims
+
+
+def test_entry_count_is_ignored_by_the_reference_mode_only(cs, orc, tmp_path):
+    """keep_values=0 stays the reference's reader, which never looks at the announced count (IO.cu:23-29)."""
+    p = tmp_path / "short.mtx"
+    p.write_text(REFUSED["fewer_entries_than_announced"])
+    r = cs.MTX_READER(str(p))
+    M, K, nnz, rp, cl, _ = orc.mtx_read(str(p))
+    assert (r.M, r.K, r.nnz) == (M, K, nnz) == (16, 16, 1) and (r.rowPtr == rp).all() and (r.cols == cl).all()
 
 
 def test_no_banner_reads_like_the_reference(cs, orc, tmp_path):

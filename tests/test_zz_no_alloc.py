@@ -57,6 +57,74 @@ def test_static_scratch_entry_point(cs, orc):
     assert plan.info["partialTileKiB"] == 0 and got.tobytes() == want.tobytes()
 
 
+def test_static_entry_point_allocates_nothing(cs):
+    """Free device memory as the driver reports it does not move across many calls, on a plan that uses the scratch."""
+    import torch
+    rng = np.random.default_rng(3)
+    M, K, N = 1024, 4096, 128
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 1500 if r in (5, 300, 900) else 6)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    plan = cs.SPMM_TC(h, N, path=cs.PATH_BRICK, mfma_shape=2)
+    assert plan.info["numAtomicChunks"] > 0
+    dB = torch.randn((K, N), device="cuda")
+    dC = torch.empty((M, N), device="cuda")
+    stream = torch.cuda.current_stream()
+    plan.run_static(dB, dC, stream=stream)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(200):
+        plan.run_static(dB, dC, stream=stream)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+
+
+def test_caller_scratch_on_two_streams(cs, orc):
+    """cute_spmm_run_scratch: one plan, two streams at the same time, each call with a buffer of its own; the bits
+    of cute_spmm_run.  Too small a buffer is refused before anything is launched."""
+    import torch
+    rng = np.random.default_rng(21)
+    M, K, N = 2048, 4096, 256
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 2500 if r % 256 == 3 else 5)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    Bs = [rng.standard_normal((K, N)).astype(np.float32) for _ in range(2)]
+    refs = [orc.spmm_csr(rp, cl, vl, B) for B in Bs]
+    for kw in (dict(path=cs.PATH_BRICK, mfma_shape=2), dict(path=cs.PATH_BRICK, mfma_shape=1), dict()):
+        plan = cs.SPMM_TC(h, N, **kw)
+        need = plan.scratch_bytes
+        assert plan.info["numAtomicChunks"] > 0 and need > 0 and (need + 1023) // 1024 == plan.info["partialTileKiB"]
+        dBs = [torch.from_numpy(B).cuda() for B in Bs]
+        want = []
+        for dB in dBs:
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            plan.run(dB, dC)
+            torch.cuda.synchronize()
+            want.append(dC.cpu().numpy())
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        scratch = [torch.empty(need, dtype=torch.uint8, device="cuda") for _ in streams]
+        outs = [torch.full((M, N), float("nan"), device="cuda") for _ in streams]
+        torch.cuda.synchronize()
+        for rep in range(10):                      # overlapping launches of the one plan
+            for i, st in enumerate(streams):
+                plan.run_scratch(dBs[i], outs[i], scratch[i], stream=st)
+        torch.cuda.synchronize()
+        for i in range(2):
+            got = outs[i].cpu().numpy()
+            assert got.tobytes() == want[i].tobytes(), (kw, i)
+            assert cs.backward_error(rp, cl, vl, Bs[i], refs[i], got) <= BERR
+        small = torch.empty(need - 16, dtype=torch.uint8, device="cuda")
+        with pytest.raises(cs.CuteError) as e:
+            plan.run_scratch(dBs[0], outs[0], small)
+        assert e.value.status == -10
+    # a plan without cut panels needs no buffer
+    plan = cs.SPMM_TC(h, N, path=cs.PATH_ROWS)
+    assert plan.scratch_bytes == 0
+    dC = torch.full((M, N), float("nan"), device="cuda")
+    plan.run_scratch(torch.from_numpy(Bs[0]).cuda(), dC, None)
+    torch.cuda.synchronize()
+    assert cs.backward_error(rp, cl, vl, Bs[0], refs[0], dC.cpu().numpy()) <= BERR
+
+
 def test_static_scratch_limit(cs):
     """A plan whose partial tiles exceed the static array is refused by the entry point, with both sizes in the message."""
     import torch
