@@ -25,7 +25,8 @@ ABI_SYMBOLS = [
     "cute_quad_build", "cute_quad_fill", "cute_quad_build_strips", "cute_quad_release", "cute_quad_census", "cute_quad_pack", "cute_hrpb_save", "cute_hrpb_load",
     "cute_partition", "cute_check_gemm_correctness", "cute_backward_error",
     "cute_gen_matrix", "cute_gen_dense",
-    "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
+    "cute_hrpb_upload", "cute_hrpb_upload_layout", "cute_hrpb_upload_device_csr", "cute_hrpb_dev_layout_sizes",
+    "cute_hrpb_dev_read_layouts", "cute_hrpb_dev_free", "cute_hrpb_dev_bytes", "cute_hrpb_dev_csr",
     "cute_spmm_plan_create", "cute_spmm_plan_info", "cute_spmm_plan_free", "cute_spmm_run", "cute_spmm_run_static",
     "cute_spmm_run_scratch", "cute_spmm_plan_scratch_bytes", "cute_device_layout",
     "cute_csr_spmm_dev", "cute_gpu_csr_spmm", "cute_spmm_time", "cute_csr_spmm_time",
@@ -182,6 +183,10 @@ def load_library():
     lib.cute_gen_dense.argtypes = [C.c_uint64, C.c_int, C.c_uint64, f32p]
     lib.cute_hrpb_upload.argtypes = [C.POINTER(cute_hrpb_host), C.POINTER(C.c_void_p)]
     lib.cute_hrpb_dev_free.argtypes = [C.c_void_p]
+    lib.cute_hrpb_upload_device_csr.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                                C.POINTER(C.c_void_p)]
+    lib.cute_hrpb_dev_layout_sizes.argtypes = [C.c_void_p, u32p, u64p, u64p, u64p, u32p]
+    lib.cute_hrpb_dev_read_layouts.argtypes = [C.c_void_p, u32p, u32p, f32p, u32p, u32p, f32p]
     lib.cute_hrpb_dev_bytes.restype = C.c_uint64
     lib.cute_hrpb_dev_bytes.argtypes = [C.c_void_p]
     lib.cute_hrpb_dev_csr.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]
@@ -465,6 +470,10 @@ class HRPB:
     def device_bytes(self):
         return load_library().cute_hrpb_dev_bytes(self._dev) if self._dev else 0
 
+    def device_layouts(self):
+        """Host copies of the layouts the device twin holds (see ``_dev_layouts``)."""
+        return _dev_layouts(self.upload(), self.M)
+
     def freeDevice(self):
         if self._dev:
             load_library().cute_hrpb_dev_free(self._dev)
@@ -552,6 +561,63 @@ def quad_pack(M, rowPtr, cols, vals, strips=False):
     _check(lib.cute_quad_pack(int(M), _ptr(rowPtr, u32p), _ptr(cols, u32p), _ptr(vals, f32p), 4 if strips else 16,
                               _ptr(groupPtr, u32p), _ptr(valBase, u64p), _ptr(recs, u32p), _ptr(packed, f32p)), "cute_quad_pack")
     return dict(groupPtr=groupPtr, recs=recs, packed=packed, stripPairs=pairs, stripVals=stored)
+
+
+def _dev_layouts(dev, M):
+    """Host copies of the layouts a device handle holds: dict with hdr [nb,32], tileVals, blockedRowPtr (brick tiles,
+    empty if not built) and recs [groups,20], quadVals, groupPtr, rowsPerList (quad lists, empty if not built)."""
+    lib = load_library()
+    nb, rows = C.c_uint32(), C.c_uint32()
+    ntv, ng, nqv = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    _check(lib.cute_hrpb_dev_layout_sizes(dev, C.byref(nb), C.byref(ntv), C.byref(ng), C.byref(nqv), C.byref(rows)),
+           "cute_hrpb_dev_layout_sizes")
+    units = M // rows.value
+    out = dict(blockedRowPtr=np.zeros(M // 16 + 1, np.uint32), hdr=np.zeros((nb.value, 32), np.uint32),
+               tileVals=np.zeros(ntv.value, np.float32), groupPtr=np.zeros(units + 1, np.uint32),
+               recs=np.zeros((ng.value, 20), np.uint32), quadVals=np.zeros(nqv.value, np.float32), rowsPerList=rows.value)
+    _check(lib.cute_hrpb_dev_read_layouts(dev, _ptr(out["blockedRowPtr"], u32p), _ptr(out["hdr"], u32p), _ptr(out["tileVals"], f32p),
+                                          _ptr(out["groupPtr"], u32p), _ptr(out["recs"], u32p), _ptr(out["quadVals"], f32p)),
+           "cute_hrpb_dev_read_layouts")
+    return out
+
+
+class DeviceHRPB:
+    """``DeviceHRPB(M, K, rowPtr, cols, vals)`` with int32 / float32 GPU tensors: the format built on the device from a
+    CSR matrix that already lives there (HRPB::HRPB + DATASTRUCT, data.cu:80-335, without the host).  Takes the place
+    of an ``HRPB`` in ``SPMM_TC(hrpb, N)``."""
+
+    def __init__(self, M, K, rowPtr, cols, vals, quad_layout=0):
+        import torch
+        for t, dt in ((rowPtr, torch.int32), (cols, torch.int32), (vals, torch.float32)):
+            if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dt and t.is_contiguous()):
+                raise TypeError("rowPtr and cols must be contiguous int32 GPU tensors, vals a contiguous float32 GPU tensor")
+        if rowPtr.numel() != int(M) + 1 or cols.numel() != vals.numel():
+            raise ValueError("rowPtr must have M+1 entries, cols and vals one per nonzero")
+        self.M, self.K, self.numNNZ = int(M), int(K), int(cols.numel())
+        self._dev = C.c_void_p()
+        _check(load_library().cute_hrpb_upload_device_csr(self.M, self.K, self.numNNZ, C.c_void_p(rowPtr.data_ptr()),
+                                                          C.c_void_p(cols.data_ptr()), C.c_void_p(vals.data_ptr()),
+                                                          int(quad_layout), C.byref(self._dev)), "cute_hrpb_upload_device_csr")
+
+    def upload(self, quad_layout=0):
+        return self._dev
+
+    def device_bytes(self):
+        return load_library().cute_hrpb_dev_bytes(self._dev)
+
+    def layouts(self):
+        return _dev_layouts(self._dev, self.M)
+
+    def freeDevice(self):
+        if self._dev:
+            load_library().cute_hrpb_dev_free(self._dev)
+            self._dev = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.freeDevice()
+        except Exception:
+            pass
 
 
 def _stream_ptr(stream):

@@ -7,6 +7,7 @@
 
 #include "common.hpp"
 #include "kernels.hip.hpp"
+#include "build_kernels.hip.hpp"
 
 using namespace cute;
 
@@ -170,8 +171,7 @@ struct cute_hrpb_dev {
     uint64_t numGroups = 0;
     std::vector<uint32_t> brp;          // host copy of blockedRowPtr
     std::vector<uint32_t> qgp;          // the quad lists' groupPtr (known from the census, before the lists are built)
-    std::vector<uint64_t> qValBase;     // index of each list unit's first stored value
-    std::vector<uint32_t> qrecsHost;    // host copy of the group records (a plan copies its chunks' first records from it)
+    std::vector<uint32_t> stripPairs;   // length of the merged column list of every 4-row strip
     uint32_t quadRows = CUTE_TM;        // rows per list unit: 16 (lockstep lists per panel) or 4 (strips)
     uint64_t quadPairs = 0;             // occupied (row group, column) pairs
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
@@ -318,74 +318,276 @@ int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out) { return cute
 
 namespace {
 
-// Brick tiles of a canonical format onto the device.
-int build_bricks(cute_hrpb_dev *d, const cute_hrpb_host *h)
+// ---- building the layouts on the device (kernels: build_kernels.hip.hpp) ----
+
+struct DevBuf {                       // device memory that lives as long as a scope
+    void *p = nullptr;
+    DevBuf() = default;
+    DevBuf(const DevBuf &) = delete;
+    DevBuf &operator=(const DevBuf &) = delete;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int alloc(uint64_t bytes)
+    {
+        HIP_TRY(hipMalloc(&p, std::max<uint64_t>(bytes, 16)));
+        return CUTE_OK;
+    }
+    template <class T> T *as() const { return static_cast<T *>(p); }
+};
+
+inline dim3 grid_of(uint64_t n) { return dim3(uint32_t((n + cute_build::kThreads - 1) / cute_build::kThreads)); }
+
+int check_launch(const char *what);
+
+// Inclusive prefix sum of n uint32 values, in place, on the default stream.
+int device_scan(uint32_t *data, uint64_t n)
 {
-    cute_hrpb_tiled t;
-    int rc = cute_hrpb_retile(h, &t);
+    if (!n) return CUTE_OK;
+    const uint64_t nb = (n + cute_build::kScanBlock - 1) / cute_build::kScanBlock;
+    if (nb > 0x7fffffffull) return CUTE_ERR_SHAPE;
+    if (nb == 1) {
+        hipLaunchKernelGGL(cute_build::scan_block_apply, dim3(1), dim3(cute_build::kThreads), 0, nullptr, data, data, n,
+                           static_cast<const uint32_t *>(nullptr));
+        return check_launch("prefix sum");
+    }
+    DevBuf sums;
+    int rc = sums.alloc(nb * sizeof(uint32_t));
     if (rc != CUTE_OK) return rc;
-    // the kernels take numVals as the position of the zero pad behind the values: the tiles must hold
-    // exactly one value per entry of the matrix, or masked lanes would read real values
-    if (t.numVals != d->numVals) { cute_hrpb_tiled_release(&t); return CUTE_ERR_FORMAT; }
-    rc = upload(&d->dHdr, t.hdr, uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS);
-    if (rc == CUTE_OK) {
-        // one wavefront of zero padding behind the values: a lane without a nonzero reads its operand there
-        std::vector<float> padded(t.numVals + 64, 0.0f);
-        if (t.numVals) std::memcpy(padded.data(), t.vals, t.numVals * sizeof(float));
-        rc = upload(&d->dVals, padded.data(), padded.size());
-    }
-    if (rc == CUTE_OK) {
-        d->bytes += uint64_t(t.numBlocks) * CUTE_TILED_HDR_WORDS * 4 + (t.numVals + 64) * 4;
-        d->haveBricks = true;
-    } else {                                  // nothing half-built stays behind: a later plan may try again
-        (void)hipFree(d->dHdr);
-        (void)hipFree(d->dVals);
-        d->dHdr = nullptr;
-        d->dVals = nullptr;
-    }
-    cute_hrpb_tiled_release(&t);
+    hipLaunchKernelGGL(cute_build::scan_block_sums, dim3(uint32_t(nb)), dim3(cute_build::kThreads), 0, nullptr, data, n, sums.as<uint32_t>());
+    rc = device_scan(sums.as<uint32_t>(), nb);
+    if (rc != CUTE_OK) return rc;
+    hipLaunchKernelGGL(cute_build::scan_block_apply, dim3(uint32_t(nb)), dim3(cute_build::kThreads), 0, nullptr, data, data, n,
+                       sums.as<const uint32_t>());
+    rc = check_launch("prefix sum");
+    // (the block sums are freed when this scope ends; hipFree waits for the kernels that read them)
     return rc;
 }
 
-// Quad lists (in the layout chosen at upload) onto the device, straight from the CSR arrays.
-int build_quads(cute_hrpb_dev *d, const uint32_t *rowPtr, const uint32_t *cols, const float *vals)
+// Where every entry of the device CSR copy stands in the (column, row) order of its panel and of its strip,
+// and the running count of distinct columns along both orders.  Checks that rows are sorted, duplicate-free
+// and inside K.  With the two vectors given, also counts active columns per panel and list pairs per strip.
+struct Census {
+    DevBuf rowOf, posP, posS, DP, DS;
+};
+
+int device_census(const cute_hrpb_dev *d, Census &c, std::vector<uint32_t> *panelCols, std::vector<uint32_t> *stripPairs)
 {
-    d->qrecsHost.assign(d->numGroups * CUTE_QUAD_RECORD_WORDS, 0u);
-    std::vector<float> packed(d->numQuadVals + 64, 0.0f);
-    int rc = cute_quad_pack(d->M, rowPtr, cols, vals, d->quadRows, d->qgp.data(), d->qValBase.data(), d->qrecsHost.data(), packed.data());
-    if (rc == CUTE_OK) rc = upload(&d->dQRecs, d->qrecsHost.data(), d->qrecsHost.size());
-    if (rc == CUTE_OK) rc = upload(&d->dQVals, packed.data(), packed.size());
-    if (rc == CUTE_OK) {
-        d->bytes += d->qrecsHost.size() * 4 + packed.size() * 4;
-        d->haveQuads = true;
-    } else {
-        (void)hipFree(d->dQRecs);
-        (void)hipFree(d->dQVals);
-        d->dQRecs = nullptr;
-        d->dQVals = nullptr;
-    }
-    return rc;
+    const uint32_t nnz = d->nnz, P = d->P;
+    if (panelCols) panelCols->assign(P, 0u);
+    if (stripPairs) stripPairs->assign(size_t(P) * 4u, 0u);
+    if (!nnz) return CUTE_OK;
+    const uint64_t bytes = uint64_t(nnz) * sizeof(uint32_t);
+    int rc = c.rowOf.alloc(bytes);
+    if (rc == CUTE_OK) rc = c.posP.alloc(bytes);
+    if (rc == CUTE_OK) rc = c.posS.alloc(bytes);
+    if (rc == CUTE_OK) rc = c.DP.alloc(bytes);
+    if (rc == CUTE_OK) rc = c.DS.alloc(bytes);
+    DevBuf err;
+    if (rc == CUTE_OK) rc = err.alloc(sizeof(int));
+    if (rc != CUTE_OK) return rc;
+    HIP_TRY(hipMemset(err.p, 0, sizeof(int)));
+    hipLaunchKernelGGL(cute_build::row_of_entries, grid_of(nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols, d->M,
+                       d->K, nnz, c.rowOf.as<uint32_t>(), err.as<int>());
+    int bad = 0;
+    HIP_TRY(hipMemcpy(&bad, err.p, sizeof(int), hipMemcpyDeviceToHost));
+    if (bad & cute_build::kErrRange) return CUTE_ERR_RANGE;
+    if (bad & cute_build::kErrUnsorted) return CUTE_ERR_UNSORTED;
+    hipLaunchKernelGGL(cute_build::entry_positions, grid_of(nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols,
+                       c.rowOf.as<const uint32_t>(), nnz, c.posP.as<uint32_t>(), c.posS.as<uint32_t>(), c.DP.as<uint32_t>(),
+                       c.DS.as<uint32_t>());
+    rc = check_launch("entry positions");
+    if (rc == CUTE_OK) rc = device_scan(c.DP.as<uint32_t>(), nnz);
+    if (rc == CUTE_OK) rc = device_scan(c.DS.as<uint32_t>(), nnz);
+    if (rc != CUTE_OK || !panelCols || !stripPairs) return rc;
+    DevBuf pc, sp;
+    rc = pc.alloc(uint64_t(P) * 4u);
+    if (rc == CUTE_OK) rc = sp.alloc(uint64_t(P) * 16u);
+    if (rc != CUTE_OK) return rc;
+    hipLaunchKernelGGL(cute_build::count_columns, grid_of(uint64_t(P) * 4u), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr,
+                       c.DP.as<const uint32_t>(), c.DS.as<const uint32_t>(), P, pc.as<uint32_t>(), sp.as<uint32_t>());
+    HIP_TRY(hipMemcpy(panelCols->data(), pc.p, uint64_t(P) * 4u, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(stripPairs->data(), sp.p, uint64_t(P) * 16u, hipMemcpyDeviceToHost));
+    return CUTE_OK;
 }
 
-// A layout the upload did not build: made from the device copy of the CSR arrays (the host arrays the
-// format borrowed may be gone by now).  which: 1 brick tiles, 2 quad lists.
-int ensure_layout(const cute_hrpb_dev *cd, int which)
+// Brick tiles from the device CSR copy: the arrays cute_hrpb_retile makes on the host, word for word.
+int build_bricks_on_device(cute_hrpb_dev *d, const Census &c)
 {
-    cute_hrpb_dev *d = const_cast<cute_hrpb_dev *>(cd);
+    const uint64_t hdr_words = uint64_t(d->nb) * CUTE_TILED_HDR_WORDS, num_vals = uint64_t(d->nnz) + 64u;
+    uint32_t *hdr = nullptr, *brp = nullptr, *pcols = nullptr;
+    float *vals = nullptr;
+    DevBuf hdr_buf, vals_buf, brp_buf, pc_buf;
+    int rc = hdr_buf.alloc(hdr_words * 4u);
+    if (rc == CUTE_OK) rc = vals_buf.alloc(num_vals * 4u);
+    if (rc == CUTE_OK) rc = brp_buf.alloc((uint64_t(d->P) + 1u) * 4u);
+    if (rc == CUTE_OK) rc = pc_buf.alloc(uint64_t(d->P) * 4u);
+    if (rc != CUTE_OK) return rc;
+    hdr = hdr_buf.as<uint32_t>(); vals = vals_buf.as<float>(); brp = brp_buf.as<uint32_t>(); pcols = pc_buf.as<uint32_t>();
+    HIP_TRY(hipMemset(hdr, 0, std::max<uint64_t>(hdr_words * 4u, 4u)));
+    HIP_TRY(hipMemset(vals + d->nnz, 0, 64u * sizeof(float)));          // one wavefront of zeros behind the values
+    HIP_TRY(hipMemcpy(brp, d->brp.data(), (uint64_t(d->P) + 1u) * 4u, hipMemcpyHostToDevice));
+    if (d->P) HIP_TRY(hipMemcpy(pcols, d->panelCols.data(), uint64_t(d->P) * 4u, hipMemcpyHostToDevice));
+    if (d->nnz) {
+        hipLaunchKernelGGL(cute_build::brick_scatter, grid_of(d->nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols,
+                           d->dCsrVals, c.rowOf.as<const uint32_t>(), c.posP.as<const uint32_t>(), c.DP.as<const uint32_t>(), brp,
+                           d->nnz, hdr, vals);
+        hipLaunchKernelGGL(cute_build::brick_finish, grid_of(d->nb), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, brp, pcols,
+                           d->P, d->nb, hdr);
+        rc = check_launch("brick tiles");
+        if (rc != CUTE_OK) return rc;
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    d->dHdr = hdr; hdr_buf.p = nullptr;
+    d->dVals = vals; vals_buf.p = nullptr;
+    d->bytes += hdr_words * 4u + num_vals * 4u;
+    d->haveBricks = true;
+    return CUTE_OK;
+}
+
+// Quad lists (in the layout the census chose) from the device CSR copy: the arrays cute_quad_pack makes.
+int build_quads_on_device(cute_hrpb_dev *d, const Census &c)
+{
+    const uint64_t G = d->numGroups;
+    const uint32_t U = uint32_t(d->qgp.size() - 1);
+    const bool strips = d->quadRows == 4;
+    DevBuf recs_buf, qgp_buf, sp_buf, counts_buf, vals_buf;
+    int rc = recs_buf.alloc(G * CUTE_QUAD_RECORD_WORDS * 4u);
+    if (rc == CUTE_OK) rc = qgp_buf.alloc(d->qgp.size() * 4u);
+    if (rc == CUTE_OK) rc = sp_buf.alloc(d->stripPairs.size() * 4u);
+    if (rc == CUTE_OK) rc = counts_buf.alloc(G * 4u);
+    if (rc != CUTE_OK) return rc;
+    uint32_t *recs = recs_buf.as<uint32_t>(), *qgp = qgp_buf.as<uint32_t>(), *sp = sp_buf.as<uint32_t>(), *counts = counts_buf.as<uint32_t>();
+    HIP_TRY(hipMemset(recs, 0, std::max<uint64_t>(G * CUTE_QUAD_RECORD_WORDS * 4u, 4u)));
+    HIP_TRY(hipMemcpy(qgp, d->qgp.data(), d->qgp.size() * 4u, hipMemcpyHostToDevice));
+    if (!d->stripPairs.empty()) HIP_TRY(hipMemcpy(sp, d->stripPairs.data(), d->stripPairs.size() * 4u, hipMemcpyHostToDevice));
+    uint32_t stored = 0;
+    if (G) {
+#define CUTE_BUILD_QUADS(S)                                                                                                          \
+    hipLaunchKernelGGL(cute_build::quad_scatter<S>, grid_of(d->nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols,     \
+                       d->dCsrVals, c.rowOf.as<const uint32_t>(), c.posS.as<const uint32_t>(), c.DS.as<const uint32_t>(), qgp, d->nnz, \
+                       recs);                                                                                                        \
+    hipLaunchKernelGGL(cute_build::quad_groups<S>, grid_of(G), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols, qgp, U, sp, \
+                       uint32_t(G), recs, counts)
+        if (strips) { CUTE_BUILD_QUADS(true); } else { CUTE_BUILD_QUADS(false); }
+#undef CUTE_BUILD_QUADS
+        rc = check_launch("quad lists");
+        if (rc == CUTE_OK) rc = device_scan(counts, G);
+        if (rc != CUTE_OK) return rc;
+        hipLaunchKernelGGL(cute_build::quad_first_values, grid_of(G), dim3(cute_build::kThreads), 0, nullptr, counts, uint32_t(G), recs);
+        HIP_TRY(hipMemcpy(&stored, counts + (G - 1u), sizeof(uint32_t), hipMemcpyDeviceToHost));
+    }
+    rc = vals_buf.alloc((uint64_t(stored) + 64u) * 4u);
+    if (rc != CUTE_OK) return rc;
+    float *packed = vals_buf.as<float>();
+    HIP_TRY(hipMemset(packed, 0, (uint64_t(stored) + 64u) * 4u));
+    if (G && d->nnz) {
+        if (strips)
+            hipLaunchKernelGGL(cute_build::quad_values<true>, grid_of(d->nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCsrVals,
+                               c.rowOf.as<const uint32_t>(), c.posS.as<const uint32_t>(), c.DS.as<const uint32_t>(), qgp, d->nnz, recs, packed);
+        else
+            hipLaunchKernelGGL(cute_build::quad_values<false>, grid_of(d->nnz), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCsrVals,
+                               c.rowOf.as<const uint32_t>(), c.posS.as<const uint32_t>(), c.DS.as<const uint32_t>(), qgp, d->nnz, recs, packed);
+        rc = check_launch("quad values");
+        if (rc != CUTE_OK) return rc;
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    d->numQuadVals = stored;
+    d->dQRecs = recs; recs_buf.p = nullptr;
+    d->dQVals = packed; vals_buf.p = nullptr;
+    d->bytes += G * CUTE_QUAD_RECORD_WORDS * 4u + (uint64_t(stored) + 64u) * 4u;
+    d->haveQuads = true;
+    return CUTE_OK;
+}
+
+// A layout the upload did not build: made on the device from the device copy of the CSR arrays (the host
+// arrays the format borrowed may be gone by now).  which: 1 brick tiles, 2 quad lists.
+int ensure_layout(cute_hrpb_dev *d, int which)
+{
     std::lock_guard<std::mutex> guard(d->lock);
     if (which == 1 ? d->haveBricks : d->haveQuads) return CUTE_OK;
-    std::vector<uint32_t> rowPtr(size_t(d->M) + 1), cols(std::max<uint32_t>(d->nnz, 1u));
-    std::vector<float> vals(std::max<uint32_t>(d->nnz, 1u));
-    HIP_TRY(hipMemcpy(rowPtr.data(), d->dRowPtr, rowPtr.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
-    if (d->nnz) {
-        HIP_TRY(hipMemcpy(cols.data(), d->dCols, size_t(d->nnz) * sizeof(uint32_t), hipMemcpyDeviceToHost));
-        HIP_TRY(hipMemcpy(vals.data(), d->dCsrVals, size_t(d->nnz) * sizeof(float), hipMemcpyDeviceToHost));
+    Census c;
+    int rc = device_census(d, c, nullptr, nullptr);
+    if (rc != CUTE_OK) return rc;
+    return which == 1 ? build_bricks_on_device(d, c) : build_quads_on_device(d, c);
+}
+
+// Group counts of the quad lists from the list length of every strip; picks lockstep lists unless they would
+// be mostly padding (a few very long rows stretch the lists of their panel neighbours): then one list per strip.
+int finish_quad_census(cute_hrpb_dev *d, std::vector<uint32_t> &strip_pairs, int quad_layout)
+{
+    const uint32_t S = d->M / 4;
+    uint64_t pairs = 0, lock_groups = 0;
+    for (uint32_t p = 0; p < d->P; ++p) {
+        uint32_t longest = 0;
+        for (uint32_t l = 0; l < 4; ++l) { longest = std::max(longest, strip_pairs[4 * p + l]); pairs += strip_pairs[4 * p + l]; }
+        lock_groups += (longest + 3) / 4;
     }
-    if (which == 2) return build_quads(d, rowPtr.data(), cols.data(), vals.data());
-    cute_hrpb_host h;
-    int rc = cute_hrpb_build(d->M, d->K, rowPtr.data(), cols.data(), vals.data(), &h);
-    if (rc == CUTE_OK) rc = build_bricks(d, &h);
-    cute_hrpb_host_release(&h);
+    if (quad_layout == 0) quad_layout = (lock_groups && double(pairs) < 0.6 * 16.0 * double(lock_groups)) ? 2 : 1;
+    d->quadRows = quad_layout == 2 ? 4u : CUTE_TM;
+    d->quadPairs = pairs;
+    const uint32_t per_unit = d->quadRows / 4, U = S / per_unit;
+    d->qgp.assign(size_t(U) + 1, 0u);
+    uint64_t groups = 0;
+    for (uint32_t u = 0; u < U; ++u) {
+        uint32_t longest = 0;
+        for (uint32_t l = 0; l < per_unit; ++l) longest = std::max(longest, strip_pairs[u * per_unit + l]);
+        groups += per_unit == 4 ? (longest + 3) / 4 : (longest + 15) / 16;
+        if (groups > 0xffffffffull / 64) return CUTE_ERR_SHAPE;
+        d->qgp[u + 1] = uint32_t(groups);
+    }
+    d->numGroups = groups;
+    d->stripPairs.swap(strip_pairs);
+    return CUTE_OK;
+}
+
+// Which MFMA layout would the planner's default rules use for this matrix (see cute_spmm_plan_create)?
+// 0: none (every panel would go to the row kernel), 1 brick tiles, 2 quad lists.
+int default_layout(const cute_hrpb_dev *d, uint64_t cache_bytes)
+{
+    const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
+    uint64_t slots = 0, bricks = 0, blocks = 0;
+    for (uint32_t q = 0; q < d->P; ++q) {
+        if (d->brp[q + 1] == d->brp[q]) continue;
+        const uint32_t list_slots = (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
+        const uint32_t fetches = std::max(d->panelCols[q], list_slots);
+        if (float(d->panelNnz[q]) < kMinReuse * float(fetches) && d->panelMaxRow[q] <= kMaxRowForRows) continue;   // row kernel
+        slots += list_slots;
+        bricks += (d->panelCols[q] + 3u) / 4u;
+        blocks += d->brp[q + 1] - d->brp[q];
+    }
+    if (!bricks) return 0;
+    // (the width is not known yet: 128 columns stand in for it)
+    return choose_mfma_shape(slots, bricks, blocks, uint64_t(d->K) + d->M, d->nnz, 128u, 0u, cache_bytes);
+}
+
+// The common tail of both uploads.  d holds the device copy of the CSR arrays, rowPtr is a host copy of the row
+// pointers (checked: ascending from 0 to nnz).  Counts active columns per panel and list pairs per strip on the
+// device, derives the planner's per-panel statistics, and builds the one MFMA layout the planner's default
+// rules would use for this matrix (none when every panel would go to the row kernel).
+int finish_upload(cute_hrpb_dev *d, const uint32_t *rowPtr, int quad_layout, const DeviceContext &c)
+{
+    Census cen;
+    std::vector<uint32_t> strip_pairs;
+    int rc = device_census(d, cen, &d->panelCols, &strip_pairs);
+    if (rc != CUTE_OK) return rc;
+    d->brp.assign(size_t(d->P) + 1, 0u);
+    d->panelNnz.resize(d->P);
+    d->panelMaxRow.resize(d->P);
+    uint64_t blocks = 0;
+    for (uint32_t p = 0; p < d->P; ++p) {
+        d->panelNnz[p] = rowPtr[(p + 1) * CUTE_TM] - rowPtr[p * CUTE_TM];
+        uint32_t longest = 0;
+        for (uint32_t r = p * CUTE_TM; r < (p + 1) * CUTE_TM; ++r) longest = std::max(longest, rowPtr[r + 1] - rowPtr[r]);
+        d->panelMaxRow[p] = longest;
+        blocks += (d->panelCols[p] + CUTE_TK - 1) / CUTE_TK;
+        if (blocks > 0xffffffffull / CUTE_TILED_HDR_WORDS) return CUTE_ERR_SHAPE;
+        d->brp[p + 1] = uint32_t(blocks);
+    }
+    d->nb = uint32_t(blocks);
+    rc = finish_quad_census(d, strip_pairs, quad_layout);
+    if (rc != CUTE_OK) return rc;
+    const int which = default_layout(d, c.cache_bytes);
+    if (which == 2) rc = build_quads_on_device(d, cen);
+    else if (which == 1) rc = build_bricks_on_device(d, cen);
     return rc;
 }
 
@@ -399,88 +601,90 @@ int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_
     *out = nullptr;
     const DeviceContext &c = context();
     if (c.status != CUTE_OK) return c.status;
+    if (h->M == 0 || h->M % CUTE_TM || h->K % CUTE_TK) return CUTE_ERR_SHAPE;
     cute_hrpb_dev *d = new cute_hrpb_dev;
     d->M = h->M;
     d->K = h->K;
     d->nnz = h->nnz;
     d->P = h->numRowPanels;
-    d->nb = h->numBlocks;
     d->numVals = h->nnz;                     // the brick tiles store every entry of the matrix once
-    d->brp.assign(h->blockedRowPtr, h->blockedRowPtr + h->numRowPanels + 1);
-    d->panelNnz.resize(d->P);
-    d->panelCols.resize(d->P);
-    d->panelMaxRow.resize(d->P);
-    for (uint32_t p = 0; p < d->P; ++p) {
-        d->panelNnz[p] = h->rowPtr[(p + 1) * CUTE_TM] - h->rowPtr[p * CUTE_TM];
-        uint32_t longest = 0;
-        for (uint32_t r = p * CUTE_TM; r < (p + 1) * CUTE_TM; ++r) longest = std::max(longest, h->rowPtr[r + 1] - h->rowPtr[r]);
-        d->panelMaxRow[p] = longest;
-        // active columns: the panel's list is ascending and zero-padded to whole blocks
-        const uint32_t nblk = d->brp[p + 1] - d->brp[p];
-        uint32_t live = 0;
-        if (nblk) {
-            const uint32_t *last = h->activeCols + uint64_t(d->brp[p + 1] - 1) * CUTE_TK;
-            uint32_t used = CUTE_TK;
-            while (used > 1 && last[used - 1] == 0) --used;
-            live = (nblk - 1) * CUTE_TK + used;
-        }
-        d->panelCols[p] = live;
-    }
     int rc = upload(&d->dRowPtr, h->rowPtr, uint64_t(h->M) + 1);
     if (rc == CUTE_OK) rc = upload(&d->dCols, h->cols, h->nnz);
     if (rc == CUTE_OK) rc = upload(&d->dCsrVals, h->vals, h->nnz);
     d->bytes = (uint64_t(h->M) + 1) * 4 + uint64_t(h->nnz) * 8;
-    // Sizes of the quad lists from one sweep over the strips.  Lockstep lists unless they would be mostly padding
-    // (a few very long rows stretch the lists of their panel neighbours): then one list per 4-row strip.
-    const uint32_t S = d->M / 4;
-    std::vector<uint32_t> strip_pairs(S), strip_vals(S);
-    if (rc == CUTE_OK) rc = cute_quad_census(h->M, h->rowPtr, h->cols, h->vals, strip_pairs.data(), strip_vals.data());
-    if (rc == CUTE_OK) {
-        uint64_t pairs = 0, lock_groups = 0;
-        for (uint32_t p = 0; p < d->P; ++p) {
-            uint32_t longest = 0;
-            for (uint32_t l = 0; l < 4; ++l) { longest = std::max(longest, strip_pairs[4 * p + l]); pairs += strip_pairs[4 * p + l]; }
-            lock_groups += (longest + 3) / 4;
-        }
-        if (quad_layout == 0) quad_layout = (lock_groups && double(pairs) < 0.6 * 16.0 * double(lock_groups)) ? 2 : 1;
-        d->quadRows = quad_layout == 2 ? 4u : CUTE_TM;
-        d->quadPairs = pairs;
-        const uint32_t per_unit = d->quadRows / 4, U = S / per_unit;
-        d->qgp.assign(size_t(U) + 1, 0u);
-        d->qValBase.assign(size_t(U) + 1, 0u);
-        uint64_t groups = 0, stored = 0;
-        for (uint32_t u = 0; u < U && rc == CUTE_OK; ++u) {
-            uint32_t longest = 0;
-            d->qValBase[u] = stored;
-            for (uint32_t l = 0; l < per_unit; ++l) { longest = std::max(longest, strip_pairs[u * per_unit + l]); stored += strip_vals[u * per_unit + l]; }
-            groups += per_unit == 4 ? (longest + 3) / 4 : (longest + 15) / 16;
-            if (groups > 0xffffffffull / 64) rc = CUTE_ERR_SHAPE;
-            d->qgp[u + 1] = uint32_t(groups);
-        }
-        d->qValBase[U] = stored;
-        d->numGroups = groups;
-        d->numQuadVals = stored;
-    }
-    if (rc == CUTE_OK) {
-        // Which MFMA layout would the planner's default rules use (see cute_spmm_plan_create)?  Build that one now.
-        const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
-        uint64_t slots = 0, bricks = 0, blocks = 0;
-        for (uint32_t q = 0; q < d->P; ++q) {
-            if (d->brp[q + 1] == d->brp[q]) continue;
-            const uint32_t list_slots = (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
-            const uint32_t fetches = std::max(d->panelCols[q], list_slots);
-            if (float(d->panelNnz[q]) < kMinReuse * float(fetches) && d->panelMaxRow[q] <= kMaxRowForRows) continue;   // row kernel
-            slots += list_slots;
-            bricks += (d->panelCols[q] + 3u) / 4u;
-            blocks += d->brp[q + 1] - d->brp[q];
-        }
-        // (the width is not known yet: 128 columns stand in for it)
-        if (bricks)
-            rc = choose_mfma_shape(slots, bricks, blocks, uint64_t(d->K) + d->M, d->nnz, 128u, 0u, c.cache_bytes) == 2
-                     ? build_quads(d, h->rowPtr, h->cols, h->vals) : build_bricks(d, h);
-    }
+    if (rc == CUTE_OK) rc = finish_upload(d, h->rowPtr, quad_layout, c);
+    // the device counted the active columns itself: it must have found the blocks the canonical format has
+    if (rc == CUTE_OK && (d->nb != h->numBlocks || std::memcmp(d->brp.data(), h->blockedRowPtr, d->brp.size() * sizeof(uint32_t)) != 0))
+        rc = CUTE_ERR_FORMAT;
     if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
     *out = d;
+    return CUTE_OK;
+}
+
+// The device-side counterpart of HRPB::HRPB + DATASTRUCT (data.cu:80-335, timed at run.cu:17-20) for a CSR
+// matrix that already lives on the device: the handle keeps its own copy of the three arrays (device to
+// device), the layouts are built by kernels, and only per-panel and per-strip counts (and the row pointers,
+// for the planner's per-panel statistics) travel to the host.
+int cute_hrpb_upload_device_csr(uint32_t M, uint32_t K, uint32_t nnz, const uint32_t *dRowPtr, const uint32_t *dCols,
+                                const float *dVals, int quad_layout, cute_hrpb_dev **out)
+{
+    if (!out || !dRowPtr || (nnz && (!dCols || !dVals)) || quad_layout < 0 || quad_layout > 2) return CUTE_ERR_ARG;
+    *out = nullptr;
+    if (M == 0 || K == 0 || M % CUTE_TM || K % CUTE_TK) return CUTE_ERR_SHAPE;
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    // the row pointers come to the host first: everything on the device indexes through them
+    std::vector<uint32_t> rowPtr(size_t(M) + 1);
+    HIP_TRY(hipMemcpy(rowPtr.data(), dRowPtr, rowPtr.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    if (rowPtr[0] != 0 || rowPtr[M] != nnz) return CUTE_ERR_RANGE;
+    for (uint32_t r = 0; r < M; ++r)
+        if (rowPtr[r + 1] < rowPtr[r]) return CUTE_ERR_RANGE;
+    cute_hrpb_dev *d = new cute_hrpb_dev;
+    d->M = M; d->K = K; d->nnz = nnz; d->P = M / CUTE_TM;
+    d->numVals = nnz;
+    auto clone = [&](auto **dst, const auto *src, uint64_t count) -> int {
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), std::max<uint64_t>(count, 1) * 4u));
+        if (count) HIP_TRY(hipMemcpy(*dst, src, count * 4u, hipMemcpyDeviceToDevice));
+        return CUTE_OK;
+    };
+    int rc = clone(&d->dRowPtr, dRowPtr, uint64_t(M) + 1);
+    if (rc == CUTE_OK) rc = clone(&d->dCols, dCols, nnz);
+    if (rc == CUTE_OK) rc = clone(&d->dCsrVals, dVals, nnz);
+    d->bytes = (uint64_t(M) + 1) * 4 + uint64_t(nnz) * 8;
+    if (rc == CUTE_OK) rc = finish_upload(d, rowPtr.data(), quad_layout, c);
+    if (rc != CUTE_OK) { cute_hrpb_dev_free(d); return rc; }
+    *out = d;
+    return CUTE_OK;
+}
+
+// Sizes and host copies of what a device handle holds, for inspection and tests.  Layouts that were not built
+// have size 0; pass nullptr for arrays that are not wanted.
+int cute_hrpb_dev_layout_sizes(const cute_hrpb_dev *d, uint32_t *numBlocks, uint64_t *numTileVals, uint64_t *numGroups,
+                               uint64_t *numQuadVals, uint32_t *rowsPerList)
+{
+    if (!d) return CUTE_ERR_ARG;
+    if (numBlocks) *numBlocks = d->haveBricks ? d->nb : 0u;
+    if (numTileVals) *numTileVals = d->haveBricks ? d->numVals : 0u;
+    if (numGroups) *numGroups = d->haveQuads ? d->numGroups : 0u;
+    if (numQuadVals) *numQuadVals = d->haveQuads ? d->numQuadVals : 0u;
+    if (rowsPerList) *rowsPerList = d->quadRows;
+    return CUTE_OK;
+}
+
+int cute_hrpb_dev_read_layouts(const cute_hrpb_dev *d, uint32_t *blockedRowPtr, uint32_t *hdr, float *tileVals, uint32_t *groupPtr,
+                               uint32_t *recs, float *quadVals)
+{
+    if (!d) return CUTE_ERR_ARG;
+    if (blockedRowPtr) std::memcpy(blockedRowPtr, d->brp.data(), d->brp.size() * sizeof(uint32_t));
+    if (groupPtr) std::memcpy(groupPtr, d->qgp.data(), d->qgp.size() * sizeof(uint32_t));
+    if (d->haveBricks) {
+        if (hdr && d->nb) HIP_TRY(hipMemcpy(hdr, d->dHdr, uint64_t(d->nb) * CUTE_TILED_HDR_WORDS * 4u, hipMemcpyDeviceToHost));
+        if (tileVals && d->numVals) HIP_TRY(hipMemcpy(tileVals, d->dVals, d->numVals * 4u, hipMemcpyDeviceToHost));
+    }
+    if (d->haveQuads) {
+        if (recs && d->numGroups) HIP_TRY(hipMemcpy(recs, d->dQRecs, d->numGroups * CUTE_QUAD_RECORD_WORDS * 4u, hipMemcpyDeviceToHost));
+        if (quadVals && d->numQuadVals) HIP_TRY(hipMemcpy(quadVals, d->dQVals, d->numQuadVals * 4u, hipMemcpyDeviceToHost));
+    }
     return CUTE_OK;
 }
 
@@ -515,7 +719,7 @@ int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out)
 // spmm.cu:11-101 and the occupancy table of spmm.cu:290-690 describe NVIDIA parts; here
 // the shape follows from wave64 MFMA tiles (16 lanes x VEC columns per group) and the slot
 // count from the CU count of the device.
-int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn, cute_spmm_plan **out)
+int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn, cute_spmm_plan **out)
 {
     if (!d || !out) return CUTE_ERR_ARG;
     *out = nullptr;
@@ -801,16 +1005,16 @@ int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunable
     if (rc == CUTE_OK) rc = upload(&p->dChunks, chunks.data(), chunks.size());
     if (rc == CUTE_OK && p->shape == 2 && !chunks.empty()) {
         // one 128-byte head per work item: its descriptor and a copy of its first group's record, so that a
-        // wavefront can ask for its first B rows after one scalar fetch instead of two dependent ones
-        std::vector<uint32_t> heads(chunks.size() * size_t(cute_dev::kQuadHeadWords), 0u);
-        for (size_t i = 0; i < chunks.size(); ++i) {
-            uint32_t *hd = heads.data() + i * cute_dev::kQuadHeadWords;
-            hd[0] = chunks[i].x; hd[1] = chunks[i].y; hd[2] = chunks[i].z; hd[3] = chunks[i].w;
-            if (chunks[i].x < chunks[i].y)               // an empty chunk (a strip without pairs) keeps a zero record
-                std::memcpy(hd + 4, d->qrecsHost.data() + size_t(chunks[i].x) * cute_dev::kQuadRecordWords,
-                            cute_dev::kQuadRecordWords * sizeof(uint32_t));
+        // wavefront can ask for its first B rows after one scalar fetch instead of two dependent ones; gathered
+        // on the device, where the records are
+        const uint64_t words = uint64_t(chunks.size()) * cute_dev::kQuadHeadWords;
+        if (hipMalloc(reinterpret_cast<void **>(&p->dHeads), words * sizeof(uint32_t)) != hipSuccess) rc = CUTE_ERR_NOMEM;
+        if (rc == CUTE_OK) {
+            hipLaunchKernelGGL(cute_build::quad_heads, grid_of(words), dim3(cute_build::kThreads), 0, nullptr, p->dChunks,
+                               uint32_t(chunks.size()), d->dQRecs, uint32_t(cute_dev::kQuadHeadWords), p->dHeads);
+            rc = check_launch("quad heads");
+            if (rc == CUTE_OK && hipStreamSynchronize(nullptr) != hipSuccess) rc = CUTE_ERR_HIP;
         }
-        rc = upload(&p->dHeads, heads.data(), heads.size());
     }
     if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
     p->unitRows = CUTE_TM / upp;

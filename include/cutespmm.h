@@ -333,15 +333,34 @@ float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, cons
  * (data.cu:327-334) and HRPB::freeDevice (data.cu:336-339).  Uploads the CSR arrays (the row
  * kernel's input) and the one MFMA layout the planner's default rules would use for this matrix --
  * brick tiles or quad lists, or neither if every panel would go to the row kernel; a plan that asks
- * for the other layout builds it then, from the device copy of the CSR arrays.
+ * for the other layout builds it then, on the device, from the device copy of the CSR arrays.
  * ---------------------------------------------------------------------------------- */
 typedef struct cute_hrpb_dev cute_hrpb_dev;
 int cute_hrpb_upload(const cute_hrpb_host *h, cute_hrpb_dev **out);
 /* Same, with the quad-list layout forced: 0 library's choice (lockstep lists unless they would be less
  * than 60 % full), 1 four lockstep lists per 16-row panel, 2 one list per 4-row strip. */
 int cute_hrpb_upload_layout(const cute_hrpb_host *h, int quad_layout, cute_hrpb_dev **out);
+/* The same from a CSR matrix that already lives on the device (an earlier kernel's output, a framework tensor):
+ * the device-side counterpart of HRPB::HRPB + DATASTRUCT (data.cu:80-335; the reference builds on the host and
+ * times it as "preprocessing", run.cu:17-20).  dRowPtr [M+1], dCols [nnz], dVals [nnz] are device pointers; the
+ * handle keeps its own copy of them.  Preconditions are checked, not assumed: M, K multiples of 16
+ * (CUTE_ERR_SHAPE), row pointers ascending from 0 to nnz and columns below K (CUTE_ERR_RANGE), columns strictly
+ * increasing inside a row (CUTE_ERR_UNSORTED).  The layouts are built by kernels and equal, word for word, what
+ * cute_hrpb_retile and cute_quad_pack make on the host from the same matrix; only the row pointers and per-panel
+ * and per-strip counts travel to the host (the planner's statistics).  Synchronises the device. */
+int cute_hrpb_upload_device_csr(uint32_t M, uint32_t K, uint32_t nnz, const uint32_t *dRowPtr, const uint32_t *dCols,
+                                const float *dVals, int quad_layout, cute_hrpb_dev **out);
 void cute_hrpb_dev_free(cute_hrpb_dev *d);
 uint64_t cute_hrpb_dev_bytes(const cute_hrpb_dev *d); /* device bytes held */
+/* Inspection: what a device handle holds.  Sizes of the layouts that have been built (0 for one that has not):
+ * blocks and values of the brick tiles, groups and stored values of the quad lists, rows per list (16 or 4); and
+ * host copies of them -- blockedRowPtr [M/16+1], hdr [numBlocks*32], tileVals [numTileVals], groupPtr [units+1],
+ * recs [numGroups*CUTE_QUAD_RECORD_WORDS], quadVals [numQuadVals]; NULL for arrays that are not wanted.  The
+ * reference keeps host and device twins of its format as public fields (data.cu:56-72). */
+int cute_hrpb_dev_layout_sizes(const cute_hrpb_dev *d, uint32_t *numBlocks, uint64_t *numTileVals, uint64_t *numGroups,
+                               uint64_t *numQuadVals, uint32_t *rowsPerList);
+int cute_hrpb_dev_read_layouts(const cute_hrpb_dev *d, uint32_t *blockedRowPtr, uint32_t *hdr, float *tileVals,
+                               uint32_t *groupPtr, uint32_t *recs, float *quadVals);
 
 /* ------------------------------------------------------------------------------------
  * device: plan + launch.   Replaces SPMM_TC::SPMM_TC / initialize_conditions / partition
@@ -401,9 +420,11 @@ typedef struct cute_plan_info {
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;
-/* Plan creation copies its tables to the device with synchronous copies (and, if the plan is the first to
- * need an MFMA layout the upload did not build, builds that layout): call it outside stream capture. */
-int cute_spmm_plan_create(const cute_hrpb_dev *d, uint32_t N, const cute_tunables *t /* may be NULL */,
+/* Plan creation copies its tables to the device with synchronous copies, gathers the quad kernels' per-item heads
+ * with a small kernel on the default stream and waits for it, and -- if the plan is the first to need an MFMA
+ * layout the upload did not build -- builds that layout on the device, inside the format handle (which is why the
+ * handle is not const; such late builds are serialised by a lock in the handle).  Call it outside stream capture. */
+int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *t /* may be NULL */,
                           cute_spmm_plan **out);
 int cute_spmm_plan_info(const cute_spmm_plan *p, cute_plan_info *out);
 void cute_spmm_plan_free(cute_spmm_plan *p);

@@ -155,6 +155,24 @@ private:
     }
 };
 
+// The format built on the device from CSR arrays that already live there (device pointers): what the HRPB
+// constructor does on the host (data.cu:80-335), by kernels.  It has no canonical host arrays to inspect; it
+// takes the place of an HRPB in SPMM_TC(M, K, N, hrpb).
+class HRPB_DEVICE {
+public:
+    unsigned int M, K, numNNZ;
+    cute_hrpb_dev *device = nullptr;
+    HRPB_DEVICE(unsigned int M_, unsigned int K_, unsigned int nnz, const unsigned int *rowPtrDevice, const unsigned int *colsDevice,
+                const float *valsDevice, int quad_layout = 0)
+        : M(M_), K(K_), numNNZ(nnz)
+    {
+        cute::check(cute_hrpb_upload_device_csr(M, K, nnz, rowPtrDevice, colsDevice, valsDevice, quad_layout, &device), "HRPB_DEVICE");
+    }
+    ~HRPB_DEVICE() { cute_hrpb_dev_free(device); }
+    HRPB_DEVICE(const HRPB_DEVICE &) = delete;
+    HRPB_DEVICE &operator=(const HRPB_DEVICE &) = delete;
+};
+
 // spmm.cu:258-840
 class SPMM_TC {
 public:
@@ -165,6 +183,11 @@ public:
         : M(M_), N(N_), K(K_)
     {
         create(hrpb, tunables);
+    }
+    SPMM_TC(unsigned int M_, unsigned int K_, unsigned int N_, const HRPB_DEVICE &hrpb, const cute_tunables *tunables = nullptr)
+        : M(M_), N(N_), K(K_)
+    {
+        create(hrpb.device, tunables);
     }
     // The reference's own signature (spmm.cu:276; call site run.cu:45): the format is found from its
     // blockedRowPtr array, which must belong to a live HRPB object that has a device copy.
@@ -205,13 +228,14 @@ public:
 private:
     cute_spmm_plan *plan_ = nullptr;
     const cute_hrpb_dev *format_ = nullptr;
-    void create(const HRPB &hrpb, const cute_tunables *tunables)
+    void create(const HRPB &hrpb, const cute_tunables *tunables) { create(hrpb.device, tunables); }
+    void create(cute_hrpb_dev *device, const cute_tunables *tunables)
     {
-        if (!hrpb.device) throw cute::Error(CUTE_ERR_ARG, "SPMM_TC: HRPB has no device copy");
-        cute::check(cute_spmm_plan_create(hrpb.device, N, tunables, &plan_), "SPMM_TC");
+        if (!device) throw cute::Error(CUTE_ERR_ARG, "SPMM_TC: HRPB has no device copy");
+        cute::check(cute_spmm_plan_create(device, N, tunables, &plan_), "SPMM_TC");
         cute_spmm_plan_info(plan_, &info);
         numRowPanelsSplit = info.numChunks;
-        format_ = hrpb.device;
+        format_ = device;
     }
 };
 

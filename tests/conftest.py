@@ -24,3 +24,10 @@ def orc():
     import oracle
     oracle.lib()
     return oracle
+
+
+@pytest.fixture(scope="session")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch

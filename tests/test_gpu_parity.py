@@ -19,13 +19,6 @@ pytestmark = pytest.mark.gpu
 BERR = 2e-6
 
 
-@pytest.fixture(scope="module")
-def torch_cuda():
-    import torch
-    assert torch.cuda.is_available(), "these tests need the MI355X"
-    return torch
-
-
 def _run(cs, torch, h, B, **kw):
     N = B.shape[1]
     dB = torch.from_numpy(np.ascontiguousarray(B)).cuda()
