@@ -37,6 +37,7 @@ ABI_SYMBOLS = [
     "cute_blocked_ell_upload", "cute_blocked_ell_dev_free", "cute_blocked_ell_spmm",
     "cute_splitter_split", "cute_split_release", "cute_classify_blocks", "cute_sequential_spmm",
     "cute_block_stats", "cute_anxs",
+    "cute_split_by_class", "cute_hybrid_create", "cute_hybrid_get_info", "cute_hybrid_spmm", "cute_hybrid_free",
 ]
 
 u32p = C.POINTER(C.c_uint32)
@@ -116,6 +117,12 @@ class cute_blocked_ell(C.Structure):
 class cute_split(C.Structure):
     _fields_ = [("totalTiles", C.c_int32), ("numHeavyTiles", C.c_int32), ("numHeavyElems", C.c_int32),
                 ("numLightTiles", C.c_int32), ("numLightElems", C.c_int32), ("heavy", cute_coo), ("light", cute_coo)]
+
+
+class cute_hybrid_info(C.Structure):
+    _fields_ = [("tileSize", C.c_int32), ("threshold", C.c_int32), ("mode", C.c_int32), ("totalTiles", C.c_int32),
+                ("heavyTiles", C.c_int32), ("heavyElems", C.c_int32), ("lightTiles", C.c_int32), ("lightElems", C.c_int32),
+                ("ellHeight", C.c_int32), ("ellWidth", C.c_int32), ("stats", C.c_float * 4)]
 
 
 class cute_block_class(C.Structure):
@@ -227,6 +234,13 @@ def load_library():
     lib.cute_classify_blocks.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_float, C.c_float,
                                          C.POINTER(C.POINTER(cute_block_class)), C.POINTER(C.c_int64)]
     lib.cute_block_stats.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, f32p]
+    lib.cute_split_by_class.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_float, C.c_float, C.POINTER(cute_split)]
+    lib.cute_hybrid_create.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_float,
+                                       C.POINTER(C.c_void_p)]
+    lib.cute_hybrid_get_info.argtypes = [C.c_void_p, C.POINTER(cute_hybrid_info)]
+    lib.cute_hybrid_spmm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p]
+    lib.cute_hybrid_free.argtypes = [C.c_void_p]
+    lib.cute_hybrid_free.restype = None
     lib.cute_anxs.argtypes = [C.POINTER(cute_csr_i32), C.c_int32, C.c_int32, f32p]
     lib.cute_sequential_spmm.restype = C.c_float
     lib.cute_sequential_spmm.argtypes = [C.POINTER(cute_csr_i32), C.POINTER(C.c_double), C.POINTER(C.c_double),
@@ -964,6 +978,56 @@ class Splitter:
     def get_num_light_elems(self): return self._c[4]
     def get_heavyMatrix(self): return self._heavy
     def get_lightMatrix(self): return self._light
+
+
+class ClassSplitter(Splitter):
+    """The split the block classifier implies (inc/preprocess.hpp:172-283): entries of dense and 2:4-sparse blocks are
+    the heavy matrix, entries of very sparse blocks the light one.  Same getters as ``Splitter``; tiles count blocks."""
+
+    def __init__(self, A_CSR, BlockSize, deviation_threshold, underload_dominance=0.5):
+        raw, out = A_CSR._raw(), cute_split()
+        _check(load_library().cute_split_by_class(C.byref(raw), int(BlockSize), float(deviation_threshold),
+                                                  float(underload_dominance), C.byref(out)), "cute_split_by_class")
+        self._c = (out.totalTiles, out.numHeavyTiles, out.numHeavyElems, out.numLightTiles, out.numLightElems)
+        self._heavy = SparseCoo(*_coo_fields(out.heavy)[:2], *_coo_fields(out.heavy)[3:])
+        self._light = SparseCoo(*_coo_fields(out.light)[:2], *_coo_fields(out.light)[3:])
+        load_library().cute_split_release(C.byref(out))
+
+
+HYBRID_SPLITTER, HYBRID_CLASSIFIER = 0, 1
+
+
+class HybridSpMM:
+    """The hybrid of inc/SPMM.cuh:2528-2933 as one library call: heavy tiles as Blocked-ELL through the fp32 MFMA
+    kernel, the remainder as CSR through the row kernel, both into one C.  ``mode`` HYBRID_SPLITTER (tile nnz
+    threshold; 0 = chosen from the block statistics) or HYBRID_CLASSIFIER (inc/preprocess.hpp:172-193)."""
+
+    def __init__(self, A_CSR, tile_size=16, nnz_threshold=0, mode=HYBRID_SPLITTER, deviation_threshold=0.5,
+                 underload_dominance=0.5):
+        raw = A_CSR._raw()
+        self.nrows, self.ncols = A_CSR.nrows, A_CSR.ncols
+        self._h = C.c_void_p()
+        _check(load_library().cute_hybrid_create(C.byref(raw), int(tile_size), int(nnz_threshold), int(mode),
+                                                 float(deviation_threshold), float(underload_dominance), C.byref(self._h)),
+               "cute_hybrid_create")
+        info = cute_hybrid_info()
+        _check(load_library().cute_hybrid_get_info(self._h, C.byref(info)), "cute_hybrid_get_info")
+        self.info = {k: getattr(info, k) for k, _ in cute_hybrid_info._fields_ if k != "stats"}
+        self.info["stats"] = [float(x) for x in info.stats]
+
+    def spmm(self, MatB, MatC, stream=None):
+        if tuple(MatB.shape)[0] != self.ncols or tuple(MatC.shape) != (self.nrows, MatB.shape[1]):
+            raise ValueError("MatB must be [%d,N] and MatC [%d,N]" % (self.ncols, self.nrows))
+        _check(load_library().cute_hybrid_spmm(self._h, _dev_ptr(MatB), _dev_ptr(MatC), int(MatB.shape[1]), _stream_ptr(stream)),
+               "cute_hybrid_spmm")
+        return MatC
+
+    def __del__(self):
+        try:
+            if self._h:
+                load_library().cute_hybrid_free(self._h)
+        except Exception:
+            pass
 
 
 def GET_STATS(A_CSR, blocksize):

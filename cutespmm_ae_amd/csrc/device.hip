@@ -1,6 +1,7 @@
 // Device side of libcutespmm: upload, plan, launch, plain CSR kernels, timing helpers.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
 #include <mutex>
 #include <string>
@@ -18,6 +19,7 @@ thread_local std::string g_hip_error;
 // The planner's default thresholds (measured on the five benchmark matrices and on the reference's 43).
 constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
 constexpr uint32_t kMaxRowForRows = 48;     // ... unless it holds a row longer than this: one lane group would serialise it
+constexpr float kHybridFill = 0.15f;         // cute_hybrid: a tile goes to the Blocked-ELL part from this fill on (threshold 0)
 constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
 // B and C together larger than the Infinity Cache: whatever the caller does between launches, their rows come
 // from HBM.  There the brick kernel's wider row pieces (16 lanes x 16 bytes per row and column group, two groups
@@ -1189,6 +1191,14 @@ struct cute_blocked_ell_dev {
     float *dValues = nullptr;
 };
 
+struct cute_hybrid {
+    cute_hybrid_info info{};
+    uint32_t rows = 0;
+    cute_blocked_ell_dev *ell = nullptr;    // heavy tiles (absent when no tile is heavy)
+    uint32_t *dRowPtr = nullptr, *dCols = nullptr;
+    float *dVals = nullptr;                 // the remainder as CSR
+};
+
 namespace {
 template <int VEC, bool ACC>
 void launch_blocked_ell(const cute_blocked_ell_dev *d, const float *dB, float *dC, uint32_t N, hipStream_t s)
@@ -1412,6 +1422,105 @@ int cute_blocked_ell_spmm(const cute_blocked_ell_dev *d, const float *dB, float 
         else launch_blocked_ell<1, false>(d, dB, dC, N, s);
     }
     return check_launch("blocked-ELL launch");
+}
+
+// ------------------------------------------------------------------------------------------------
+// The hybrid the reference's earlier prototypes model (inc/SPMM.cuh:2528-2933 GPU_Compute_Multi_Kernel*,
+// the 2-D variant at :2898: tiles with more than THRESHOLD entries go to the tensor cores as dense tiles,
+// the rest to a plain kernel; inc/splitter.hpp and inc/preprocess.hpp:172-193 are its two split rules):
+// heavy tiles as a Blocked-ELL matrix through blocked_ell_f32 (fp32 MFMA), the remainder through the CSR
+// row kernel, both into one C.
+// ------------------------------------------------------------------------------------------------
+void cute_hybrid_free(cute_hybrid *h)
+{
+    if (!h) return;
+    cute_blocked_ell_dev_free(h->ell);
+    (void)hipFree(h->dRowPtr);
+    (void)hipFree(h->dCols);
+    (void)hipFree(h->dVals);
+    delete h;
+}
+
+int cute_hybrid_create(const cute_csr_i32 *csr, int32_t tile_size, int32_t nnz_threshold, int32_t mode, float deviation_threshold,
+                       float underload_dominance, cute_hybrid **out)
+{
+    if (!csr || !out || !csr->rowPtr || (mode != CUTE_HYBRID_SPLITTER && mode != CUTE_HYBRID_CLASSIFIER)) return CUTE_ERR_ARG;
+    *out = nullptr;
+    if (tile_size <= 0 || tile_size % 16 || csr->nrows <= 0 || csr->nrows % tile_size || csr->ncols % tile_size) return CUTE_ERR_SHAPE;
+    const DeviceContext &c = context();
+    if (c.status != CUTE_OK) return c.status;
+    cute_hybrid *h = new cute_hybrid;
+    h->info.tileSize = tile_size;
+    h->info.mode = mode;
+    h->rows = uint32_t(csr->nrows);
+    int rc = cute_block_stats(csr, tile_size, h->info.stats);
+    cute_split sp{};
+    if (rc == CUTE_OK) {
+        if (mode == CUTE_HYBRID_SPLITTER) {
+            // Threshold 0: the fill from which a tile pays for itself on the matrix cores, measured on gfx950 with this
+            // library's two kernels (16 384^2 matrices, a sparse background plus 20 000 tiles of a given fill, N = 128):
+            // tiles 10 % full lose 10 us by moving to the Blocked-ELL part (37.6 against 27.9 us), tiles 20 % full win 9 us
+            // (36.2 against 45.6), tiles 30 % full 28 us -- the break-even is near 15 % of the tile's cells.  And a heavy
+            // part that would hold less than 2 % of the entries is not worth its own launch (14 tiles of the FEM
+            // benchmark matrix: +9 us): everything then stays with the row kernel.
+            const bool automatic = nnz_threshold <= 0;
+            if (automatic) nnz_threshold = std::max(1, int32_t(std::ceil(kHybridFill * float(tile_size) * float(tile_size))));
+            rc = cute_splitter_split(csr, tile_size, nnz_threshold, &sp);
+            if (rc == CUTE_OK && automatic && sp.numHeavyElems && int64_t(sp.numHeavyElems) * 50 < int64_t(csr->nnz)) {
+                cute_split_release(&sp);
+                nnz_threshold = tile_size * tile_size + 1;
+                rc = cute_splitter_split(csr, tile_size, nnz_threshold, &sp);
+            }
+        } else {
+            rc = cute_split_by_class(csr, tile_size, deviation_threshold, underload_dominance, &sp);
+            nnz_threshold = 0;
+        }
+    }
+    h->info.threshold = nnz_threshold;
+    cute_csr_i32 heavy{}, light{};
+    cute_blocked_ell ell{};
+    if (rc == CUTE_OK) {
+        h->info.totalTiles = sp.totalTiles;
+        h->info.heavyTiles = sp.numHeavyTiles; h->info.heavyElems = sp.numHeavyElems;
+        h->info.lightTiles = sp.numLightTiles; h->info.lightElems = sp.numLightElems;
+        rc = cute_coo_to_csr(&sp.light, &light);
+    }
+    if (rc == CUTE_OK && sp.numHeavyElems) rc = cute_coo_to_csr(&sp.heavy, &heavy);
+    if (rc == CUTE_OK && sp.numHeavyElems) rc = cute_blocked_ell_build(&heavy, tile_size, &ell);
+    if (rc == CUTE_OK && sp.numHeavyElems) {
+        h->info.ellHeight = ell.height;
+        h->info.ellWidth = ell.width;
+        rc = cute_blocked_ell_upload(&ell, &h->ell);
+    }
+    if (rc == CUTE_OK) rc = upload(&h->dRowPtr, reinterpret_cast<const uint32_t *>(light.rowPtr), uint64_t(csr->nrows) + 1);
+    if (rc == CUTE_OK) rc = upload(&h->dCols, reinterpret_cast<const uint32_t *>(light.cols), uint64_t(light.nnz));
+    if (rc == CUTE_OK) rc = upload(&h->dVals, light.values, uint64_t(light.nnz));
+    cute_blocked_ell_release(&ell);
+    cute_csr_i32_release(&heavy);
+    cute_csr_i32_release(&light);
+    cute_split_release(&sp);
+    if (rc != CUTE_OK) { cute_hybrid_free(h); return rc; }
+    *out = h;
+    return CUTE_OK;
+}
+
+int cute_hybrid_get_info(const cute_hybrid *h, cute_hybrid_info *out)
+{
+    if (!h || !out) return CUTE_ERR_ARG;
+    *out = h->info;
+    return CUTE_OK;
+}
+
+// C[nrows x N] = A . B: the remainder through the row kernel (which writes every row of C), then the heavy tiles
+// added on top by the Blocked-ELL kernel; both asynchronous on `stream`, in that order.
+int cute_hybrid_spmm(const cute_hybrid *h, const float *dB, float *dC, uint32_t N, void *stream)
+{
+    if (!h || !dB || !dC) return CUTE_ERR_ARG;
+    if (N == 0) return CUTE_ERR_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC)) & 15u) return CUTE_ERR_ARG;
+    int rc = csr_launch(2, h->dRowPtr, h->dCols, h->dVals, dB, dC, h->rows, N, static_cast<hipStream_t>(stream));
+    if (rc == CUTE_OK && h->ell) rc = cute_blocked_ell_spmm(h->ell, dB, dC, N, 1, stream);
+    return rc;
 }
 
 // Shape of GPU_CSR_cuSPARSE_NEW (spmm.cu:860-960): host arrays in, host C out, one warm-up

@@ -525,6 +525,61 @@ int cute_classify_blocks(const cute_csr_i32 *a, int32_t B, float dev_thr, float 
     return CUTE_OK;
 }
 
+// The split the classifier implies (inc/preprocess.hpp:196-283 builds three containers from it): entries of
+// blocks classified dense or 2:4-sparse form the part for the matrix cores, entries of very sparse blocks the
+// remainder.  Same containers and CSR-order filling as the Splitter's.
+int cute_split_by_class(const cute_csr_i32 *a, int32_t B, float dev_thr, float dominance, cute_split *out)
+{
+    if (!csr_ok(a) || !out || B < 4 || B % 4) return CUTE_ERR_ARG;
+    std::memset(out, 0, sizeof(*out));
+    cute_block_class *cls = nullptr;
+    int64_t n = 0;
+    int rc = cute_classify_blocks(a, B, dev_thr, dominance, &cls, &n);
+    if (rc != CUTE_OK) return rc;
+    const int nbr = (a->nrows + B - 1) / B;
+    std::vector<int64_t> first(size_t(nbr) + 1, n);          // blocks are sorted by (blockRow, blockCol)
+    for (int64_t i = n - 1; i >= 0; --i) first[size_t(cls[i].blockRow)] = i;
+    for (int br = nbr - 1; br >= 0; --br) first[size_t(br)] = std::min(first[size_t(br)], first[size_t(br) + 1]);
+    out->totalTiles = int32_t(n);
+    for (int64_t i = 0; i < n; ++i) (cls[i].kind == 2 ? out->numLightTiles : out->numHeavyTiles)++;
+    std::vector<uint8_t> heavy(static_cast<size_t>(a->nnz), uint8_t(0));
+    parallel_ranges(uint64_t(nbr), 8, [&](uint64_t bb, uint64_t be, unsigned) {
+        for (uint64_t br = bb; br < be; ++br) {
+            const cute_block_class *lo = cls + first[br], *hi = cls + first[br + 1];
+            const int r1 = std::min(a->nrows, int(br + 1) * B);
+            for (int r = int(br) * B; r < r1; ++r)
+                for (int e = a->rowPtr[r]; e < a->rowPtr[r + 1]; ++e) {
+                    const int bc = a->cols[e] / B;
+                    const cute_block_class *it = std::lower_bound(lo, hi, bc, [](const cute_block_class &x, int c) { return x.blockCol < c; });
+                    heavy[size_t(e)] = (it != hi && it->blockCol == bc && it->kind != 2) ? 1 : 0;
+                }
+        }
+    });
+    std::free(cls);
+    for (uint8_t h : heavy) (h ? out->numHeavyElems : out->numLightElems)++;
+    cute_coo *dst[2] = {&out->light, &out->heavy};
+    const int cnt[2] = {out->numLightElems, out->numHeavyElems};
+    for (int k = 0; k < 2; ++k) {
+        dst[k]->dimY = a->nrows;
+        dst[k]->dimX = a->ncols;
+        dst[k]->nnz = cnt[k];
+        dst[k]->rows = alloc_array<int32_t>(size_t(cnt[k]));
+        dst[k]->cols = alloc_array<int32_t>(size_t(cnt[k]));
+        dst[k]->values = alloc_array<float>(size_t(cnt[k]));
+        if (!dst[k]->rows || !dst[k]->cols || !dst[k]->values) { cute_split_release(out); return CUTE_ERR_NOMEM; }
+    }
+    int fill[2] = {0, 0};
+    for (int r = 0; r < a->nrows; ++r)
+        for (int e = a->rowPtr[r]; e < a->rowPtr[r + 1]; ++e) {
+            const int k = heavy[size_t(e)];
+            dst[k]->rows[fill[k]] = r;
+            dst[k]->cols[fill[k]] = a->cols[e];
+            dst[k]->values[fill[k]] = a->values[e];
+            fill[k]++;
+        }
+    return CUTE_OK;
+}
+
 float cute_sequential_spmm(const cute_csr_i32 *a, const double *vals, const double *B, double *C, int32_t m, int32_t k, int32_t n)
 {
     (void)k;

@@ -312,6 +312,12 @@ typedef struct cute_block_class {  /* one non-empty blockSize^2 block, inc/prepr
 int cute_classify_blocks(const cute_csr_i32 *csr, int32_t blockSize, float deviation_threshold,
                          float underload_dominance, cute_block_class **out, int64_t *count);
 
+/* The split the classifier implies (inc/preprocess.hpp:196-283 fills three containers from it): entries of blocks
+ * classified dense or 2:4-sparse are the `heavy` part, entries of very sparse blocks the `light` part; tile counters
+ * count blocks.  Same containers as the Splitter's. */
+int cute_split_by_class(const cute_csr_i32 *csr, int32_t blockSize, float deviation_threshold, float underload_dominance,
+                        cute_split *out);
+
 /* GET_STATS, gpu_kernels.cu:1049-1137, the features its split threshold is chosen from: over the non-empty
  * blocksize^2 blocks, stats[0] = mean of nnz / distinct rows, stats[1] = mean of nnz / distinct columns,
  * stats[2] = number of blocks, stats[3] = mean of nnz / blocksize^2.  Blocks are told apart by the reference's
@@ -323,6 +329,36 @@ int cute_block_stats(const cute_csr_i32 *csr, int32_t blocksize, float stats[4])
 /* GET_ANXS, gpu_kernels.cu:1139-1186: nnz / number of distinct (band, segment) pairs; axis != 0: bands are
  * block rows and segments columns, axis == 0: bands are block columns and segments rows. */
 int cute_anxs(const cute_csr_i32 *csr, int32_t blocksize, int32_t axis, float *out);
+
+/* ------------------------------------------------------------------------------------
+ * device: the hybrid of the reference's earlier prototypes (inc/SPMM.cuh:2528-2933, GPU_Compute_Multi_Kernel*;
+ * the 2-D variant at :2898 sends tiles with more than THRESHOLD entries to the tensor cores as dense tiles and the
+ * rest to a plain kernel): a matrix split into heavy tiles, kept as a Blocked-ELL matrix and multiplied by the fp32
+ * MFMA kernel, and a remainder kept as CSR and multiplied by the row kernel; both into one C.
+ *   mode CUTE_HYBRID_SPLITTER    the Splitter's rule (inc/splitter.hpp:71-80): a tile_size^2 tile is heavy when it
+ *                                holds at least nnz_threshold entries; nnz_threshold 0: 15 % of the tile's cells, the
+ *                                break-even measured on gfx950 between this library's two kernels, and no heavy part at
+ *                                all when it would hold less than 2 % of the entries.  The block statistics the
+ *                                reference's harness chooses from (cute_block_stats) are reported in the info.
+ *   mode CUTE_HYBRID_CLASSIFIER  the classifier's rule (inc/preprocess.hpp:172-193, cute_classify_blocks): dense and
+ *                                2:4-sparse blocks are heavy, very sparse ones the remainder
+ * tile_size: a multiple of 16 that divides nrows and ncols (the harness pads first, gpu_kernels.cu:1415-1430).
+ * ---------------------------------------------------------------------------------- */
+enum { CUTE_HYBRID_SPLITTER = 0, CUTE_HYBRID_CLASSIFIER = 1 };
+typedef struct cute_hybrid_info {
+    int32_t tileSize, threshold, mode;      /* threshold: the one in use (0 in classifier mode)               */
+    int32_t totalTiles, heavyTiles, heavyElems, lightTiles, lightElems;
+    int32_t ellHeight, ellWidth;            /* Blocked-ELL shape of the heavy part (0 x 0 when there is none)  */
+    float stats[4];                         /* cute_block_stats of the whole matrix at tile_size               */
+} cute_hybrid_info;
+typedef struct cute_hybrid cute_hybrid;
+int cute_hybrid_create(const cute_csr_i32 *csr, int32_t tile_size, int32_t nnz_threshold, int32_t mode,
+                       float deviation_threshold, float underload_dominance, cute_hybrid **out);
+int cute_hybrid_get_info(const cute_hybrid *h, cute_hybrid_info *out);
+/* dB [ncols x N], dC [nrows x N]: device pointers, 16-byte aligned; C is overwritten.  Asynchronous on `stream`. */
+int cute_hybrid_spmm(const cute_hybrid *h, const float *dB, float *dC, uint32_t N, void *stream);
+void cute_hybrid_free(cute_hybrid *h);
+
 
 /* sequentioal_spmm, inc/SPMM.cuh:123-187: double-precision CPU CSR SpMM; returns ms. */
 float cute_sequential_spmm(const cute_csr_i32 *csr, const double *vals_f64, const double *B, double *C,

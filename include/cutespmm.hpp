@@ -419,6 +419,33 @@ private:
     SparseCoo<float> *heavy_ = nullptr, *light_ = nullptr;
 };
 
+// The hybrid of inc/SPMM.cuh:2528-2933 (GPU_Compute_Multi_Kernel*: dense part on the matrix cores, remainder on a
+// plain kernel) as one object: heavy tiles by the Splitter's rule (NNZThreshold 0: the library's measured default)
+// or by the block classifier's (inc/preprocess.hpp:172-193), multiplied into one C.
+class HybridSpMM {
+public:
+    cute_hybrid_info info{};
+    HybridSpMM(CSR_Matrix<float> *A_CSR, int tile_size = 16, int NNZThreshold = 0)
+    {
+        cute::check(cute_hybrid_create(&A_CSR->raw(), tile_size, NNZThreshold, CUTE_HYBRID_SPLITTER, 0.0f, 0.0f, &h_), "HybridSpMM");
+        cute_hybrid_get_info(h_, &info);
+    }
+    HybridSpMM(CSR_Matrix<float> *A_CSR, int BlockSize, float deviation_threshold, float underloadDominance)
+    {
+        cute::check(cute_hybrid_create(&A_CSR->raw(), BlockSize, 0, CUTE_HYBRID_CLASSIFIER, deviation_threshold, underloadDominance, &h_),
+                    "HybridSpMM");
+        cute_hybrid_get_info(h_, &info);
+    }
+    // dB [ncols x N], dC [nrows x N]: device pointers; asynchronous on `stream`
+    void run(const float *dB, float *dC, uint32_t N, void *stream = nullptr) { cute::check(cute_hybrid_spmm(h_, dB, dC, N, stream), "HybridSpMM::run"); }
+    ~HybridSpMM() { cute_hybrid_free(h_); }
+    HybridSpMM(const HybridSpMM &) = delete;
+    HybridSpMM &operator=(const HybridSpMM &) = delete;
+
+private:
+    cute_hybrid *h_ = nullptr;
+};
+
 // Block statistics the reference's harness chooses its split threshold from (gpu_kernels.cu:1049-1186).
 inline void GET_STATS(CSR_Matrix<float> *A_CSR, uint32_t blocksize, std::vector<float> &stats)
 {

@@ -230,6 +230,31 @@ def test_product_classifier_equals_oracle(cs, orc):
         assert got[:, 2].sum() == len(cl)
 
 
+def test_product_split_by_class_equals_oracle(cs, orc):
+    """The split the classifier implies: an entry is heavy iff its block is not "very sparse" (kind 2) by the oracle's
+    band statistics and rule (inc/preprocess.hpp:64-193 restated); heavy and light together are the matrix, in CSR order."""
+    for seed, B, thr, dom in [(30, 16, 0.5, 0.8), (31, 8, 0.25, 0.5), (32, 32, 0.1, 0.9), (33, 16, 0.9, 0.3)]:
+        M, K, rp, cl, vl = _csr_case(seed, 64, 128, 0.15)
+        csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp, cols=cl, values=vl)
+        s = cs.ClassSplitter(csr, B, thr, dom)
+        st = orc.block_stats(M, K, rp, cl, B)
+        kind = np.full(st.shape[:2], -1)
+        for br in range(st.shape[0]):
+            for bc in range(st.shape[1]):
+                n, u, o = st[br, bc]
+                if n:
+                    kind[br, bc] = orc.classify(n, u, o, B, thr, dom)
+        rows = np.repeat(np.arange(M), np.diff(rp))
+        which = kind[rows // B, cl // B] != 2
+        assert (kind[rows // B, cl // B] >= 0).all()
+        h, l = s.get_heavyMatrix(), s.get_lightMatrix()
+        assert (h.rows == rows[which]).all() and (h.cols == cl[which]).all() and (h.values == vl[which]).all()
+        assert (l.rows == rows[~which]).all() and (l.cols == cl[~which]).all() and (l.values == vl[~which]).all()
+        assert s.get_total_tiles() == (kind >= 0).sum() and s.get_num_light_tiles() == (kind == 2).sum()
+        assert s.get_num_heavy_tiles() == ((kind == 0) | (kind == 1)).sum()
+        assert s.get_num_heavy_elems() == which.sum() and s.get_num_light_elems() == (~which).sum()
+
+
 def test_product_double_spmm_equals_oracle(cs, orc):
     M, K, rp, cl, vl = _csr_case(40, 25, 33, 0.2)
     csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp, cols=cl, values=vl)

@@ -610,6 +610,58 @@ def test_split_matrix_spmm(cs, orc, torch_cuda):
     assert (dC.cpu().numpy() == orc.spmm_csr(rp, cl, vl, B)).all()
 
 
+def test_hybrid_spmm(cs, orc, torch_cuda):
+    """cute_hybrid_*: heavy tiles through the Blocked-ELL MFMA kernel, the remainder through the row kernel, one call.
+    Exact on integer-valued inputs (every sum is exact in fp32), for both split rules and for thresholds that send
+    everything, nothing and some of the matrix to the matrix cores; within tolerance on real values."""
+    torch = torch_cuda
+    rng = np.random.default_rng(78)
+    M, K, N = 256, 320, 64
+    D = np.zeros((M, K), np.float32)
+    D[rng.random((M, K)) < 0.01] = 1.0                      # light background
+    for t in rng.choice((M // 16) * (K // 16), 50, replace=False):   # some dense 16x16 tiles
+        r, c = (t // (K // 16)) * 16, (t % (K // 16)) * 16
+        D[r:r + 16, c:c + 16] = (rng.random((16, 16)) < 0.7)
+    D *= rng.integers(1, 4, D.shape)
+    rp, cl, vl = csr_from_dense(D)
+    csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp.astype(np.int32), cols=cl.astype(np.int32), values=vl)
+    B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    dB = torch.from_numpy(B).cuda()
+    seen = set()
+    for kw in (dict(), dict(nnz_threshold=1), dict(nnz_threshold=257), dict(nnz_threshold=40), dict(tile_size=32),
+               dict(mode=cs.HYBRID_CLASSIFIER, deviation_threshold=0.5, underload_dominance=0.8),
+               dict(mode=cs.HYBRID_CLASSIFIER, deviation_threshold=0.1, underload_dominance=0.5)):
+        hy = cs.HybridSpMM(csr, **kw)
+        info = hy.info
+        assert info["heavyElems"] + info["lightElems"] == len(vl) and info["heavyTiles"] + info["lightTiles"] == info["totalTiles"]
+        dC = torch.full((M, N), float("nan"), device="cuda")
+        hy.spmm(dB, dC)
+        torch.cuda.synchronize()
+        assert (dC.cpu().numpy() == ref).all(), kw
+        seen.add((info["heavyElems"] > 0, info["lightElems"] > 0))
+    assert seen == {(True, True), (True, False), (False, True)}
+    # the default threshold: 15 % of the tile's cells (measured break-even); the harness's block statistics ride along
+    hy = cs.HybridSpMM(csr)
+    st = cs.GET_STATS(csr, 16)
+    assert hy.info["threshold"] == 39 and hy.info["stats"][2] == st[2] and hy.info["stats"][3] == st[3]
+    sp = cs.Splitter(csr, 16, hy.info["threshold"])
+    assert (hy.info["heavyTiles"], hy.info["heavyElems"]) == (sp.get_num_heavy_tiles(), sp.get_num_heavy_elems())
+    # real values, a wider N that is not a multiple of the slab
+    vr = rng.standard_normal(len(vl)).astype(np.float32)
+    csr_r = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp.astype(np.int32), cols=cl.astype(np.int32), values=vr)
+    Br = rng.standard_normal((K, 100)).astype(np.float32)
+    dC = torch.full((M, 100), float("nan"), device="cuda")
+    cs.HybridSpMM(csr_r).spmm(torch.from_numpy(Br).cuda(), dC)
+    torch.cuda.synchronize()
+    assert cs.backward_error(rp, cl, vr, Br, orc.spmm_csr(rp, cl, vr, Br), dC.cpu().numpy()) <= BERR
+    # shapes the Blocked-ELL part cannot take are refused
+    odd = cs.CSR_Matrix(nrows=40, ncols=64, rowPtr=np.zeros(41, np.int32), cols=np.zeros(0, np.int32), values=np.zeros(0, np.float32))
+    with pytest.raises(cs.CuteError) as e:
+        cs.HybridSpMM(odd)
+    assert e.value.status == -2
+
+
 @pytest.mark.timeout(600)
 @pytest.mark.parametrize("cfg", [3, 4, 5])
 def test_full_size_other_configs(cs, orc, torch_cuda, cfg):
