@@ -18,6 +18,7 @@ thread_local std::string g_hip_error;
 
 // The planner's default thresholds (measured on the five benchmark matrices and on the reference's 43).
 constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
+constexpr float kWideReuse = 0.98f;          // ... the bar for products of 256 columns or more over large matrices (see cute_spmm_plan_create)
 constexpr uint32_t kMaxRowForRows = 48;     // ... unless it holds a row longer than this: one lane group would serialise it
 constexpr float kHybridFill = 0.15f;         // cute_hybrid: a tile goes to the Blocked-ELL part from this fill on (threshold 0)
 constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
@@ -736,7 +737,16 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : kMaxRowForRows;
     // An MFMA work item always spans 64 output columns; when N is narrower the row kernel wastes
     // less, so the reuse a panel must offer to earn the MFMA kernel grows (measured on N = 8..32).
-    const float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
+    float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
+    // Wide products of large matrices: the row kernel walks three dependent round trips per row (row pointers,
+    // entries, B rows), the quad kernel streams its lists two groups ahead, and with 256 columns or more and a launch
+    // several times the size of the device that depth counts for more than reuse: on 50 000 rows of 7 entries at
+    // random columns, N = 512, the quad kernel takes 93 us against 116; ncvxbqp1, mk12-b3, delaunay_n16 of the
+    // reference's matrices gain 10-20 % the same way.  There the bar drops to "the lists need no more fetches than the
+    // panel has entries" (matrices whose short lists would be mostly padding -- cat_ears_4_4, Wordnet3 -- stay with
+    // the row kernel, which is 20 % ahead on them).
+    if (t.min_reuse <= 0.0f && N >= 256u && uint64_t(d->M) * ((N + 255u) / 256u) >= 4ull * uint64_t(c.num_cus) * 32u)
+        reuse_bar = kWideReuse;
 
     cute_spmm_plan *p = new cute_spmm_plan;
     p->d = d;

@@ -422,6 +422,34 @@ def test_default_kernel_choice(cs, orc, torch_cuda):
         assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
 
 
+def test_wide_products_of_short_rows_go_to_the_quad_kernel(cs, orc, torch_cuda):
+    """50 000 rows of 7 entries at random columns: no reuse for the matrix cores to harvest, and at N = 128 the row
+    kernel keeps them; at N = 512 the launch is several times the device and the quad kernel's deeper pipeline wins
+    (93 against 116 us), so the planner sends the panels there.  Same product either way."""
+    rng = np.random.default_rng(3)
+    M = K = 50000 // 16 * 16
+    cols = np.sort(rng.integers(0, K - 64, (M, 7)), axis=1)
+    cols += np.arange(7)[None, :] * 8 * (np.diff(cols, axis=1, prepend=-1) == 0).cumsum(1)      # make equal neighbours distinct
+    cols = np.sort(cols, axis=1)
+    keep = (np.diff(cols, axis=1) > 0).all(1)
+    cols[~keep] = np.arange(7)[None, :] * 3 + 5                                                 # the rare leftover rows
+    rp = (np.arange(M + 1) * 7).astype(np.uint32)
+    cl, vl = cols.ravel().astype(np.uint32), rng.standard_normal(M * 7).astype(np.float32)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    narrow = cs.SPMM_TC(h, 128)
+    assert narrow.kernel_name == "csr_rows_batched" and narrow.info["numChunks"] == 0
+    B = rng.standard_normal((K, 512)).astype(np.float32)
+    out, wide = _run(cs, torch_cuda, h, B)
+    assert wide.info["mfmaShape"] == 2 and wide.kernel_name.startswith("hrpb_quad"), wide.info
+    assert wide.info["numBrickPanels"] > 0.9 * (M // 16)
+    ref = orc.spmm_csr(rp, cl, vl, B)
+    assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
+    same, rows = _run(cs, torch_cuda, h, B, path=cs.PATH_ROWS)
+    assert cs.backward_error(rp, cl, vl, B, ref, same) <= BERR
+    # a caller's own bar overrides the rule
+    assert cs.SPMM_TC(h, 512, min_reuse=1.25).info["numChunks"] == 0
+
+
 def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
     """An upload sends the CSR arrays and the one MFMA layout the planner's default rules would use (none when every
     panel would go to the row kernel); a plan that asks for the other one builds it then, from the device copy of the
