@@ -80,7 +80,7 @@ class cute_quad_lists(C.Structure):
 class cute_tunables(C.Structure):
     _fields_ = [("path", C.c_int32), ("precision", C.c_int32), ("min_reuse", C.c_float), ("slots", C.c_uint32),
                 ("max_chunk_blocks", C.c_uint32), ("brick_groups", C.c_uint32), ("pipeline", C.c_uint32), ("mfma_shape", C.c_uint32), ("max_row_nnz", C.c_uint32),
-                ("chunk_order", C.c_uint32), ("operand_residency", C.c_uint32), ("reserved", C.c_uint32 * 1)]
+                ("chunk_order", C.c_uint32), ("operand_residency", C.c_uint32), ("hub_rows", C.c_uint32)]
 
 
 class cute_plan_info(C.Structure):
@@ -88,7 +88,7 @@ class cute_plan_info(C.Structure):
                 ("numAtomicChunks", C.c_uint32), ("numBrickPanels", C.c_uint32), ("numRowPanelsSparse", C.c_uint32),
                 ("numEmptyPanels", C.c_uint32), ("slots", C.c_uint32), ("precision", C.c_uint32),
                 ("path", C.c_uint32), ("mfmaShape", C.c_uint32), ("pipeline", C.c_uint32),
-                ("fusedLaunch", C.c_uint32), ("dealtChunks", C.c_uint32), ("partialTileKiB", C.c_uint32)]
+                ("fusedLaunch", C.c_uint32), ("dealtChunks", C.c_uint32), ("partialTileKiB", C.c_uint32), ("hubRows", C.c_uint32)]
 
 
 i32p = C.POINTER(C.c_int32)
@@ -645,13 +645,13 @@ class SPMM_TC:
     (spmm.cu:823-839) on torch's current stream.  MatB [K,N], MatC [M,N] float32 GPU tensors."""
 
     def __init__(self, hrpb, N, path=PATH_AUTO, precision=PREC_FP32, min_reuse=0.0, slots=0, max_chunk_blocks=0,
-                 brick_groups=0, pipeline=0, mfma_shape=0, max_row_nnz=0, chunk_order=0, operand_residency=0):
+                 brick_groups=0, pipeline=0, mfma_shape=0, max_row_nnz=0, chunk_order=0, operand_residency=0, hub_rows=0):
         self.hrpb = hrpb
         self.M, self.K, self.N = hrpb.M, hrpb.K, int(N)
         self._plan = C.c_void_p()
         t = cute_tunables(path=path, precision=precision, min_reuse=min_reuse, slots=slots,
                           max_chunk_blocks=max_chunk_blocks, brick_groups=brick_groups, pipeline=pipeline, mfma_shape=mfma_shape,
-                          max_row_nnz=max_row_nnz, chunk_order=chunk_order, operand_residency=operand_residency)
+                          max_row_nnz=max_row_nnz, chunk_order=chunk_order, operand_residency=operand_residency, hub_rows=hub_rows)
         _check(load_library().cute_spmm_plan_create(hrpb.upload(), self.N, C.byref(t), C.byref(self._plan)),
                "cute_spmm_plan_create")
         info = cute_plan_info()
@@ -659,6 +659,7 @@ class SPMM_TC:
         self.info = {k: getattr(info, k) for k, _ in cute_plan_info._fields_ if k != "reserved"}
         self.numRowPanelsSplit = info.numChunks
         self.kernel_name = ("csr_rows_batched" if info.numChunks == 0 else
+                            "hrpb_quad_hub_f32" if info.hubRows else
                             ("hrpb_quad_rows_f32" if info.fusedLaunch else "hrpb_quad_f32") if info.mfmaShape == 2 else
                             "hrpb_brick_rows_f32" if info.fusedLaunch else
                             "hrpb_brick_bf16x3" if info.precision == PREC_BF16X3 else

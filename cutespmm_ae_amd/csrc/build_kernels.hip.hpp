@@ -339,4 +339,28 @@ __global__ __launch_bounds__(kThreads) void quad_heads(const uint4 *__restrict__
     heads[id] = v;
 }
 
+// Hub plans (hrpb_quad_hub_f32): how often every column occurs in the quad records, and a copy of the records in
+// which the columns that have a slot in the LDS table of hub rows (slot_of[col] != ~0u) name that slot instead.
+__global__ __launch_bounds__(kThreads) void count_record_columns(const uint32_t *__restrict__ recs, uint64_t numGroups,
+                                                                 uint32_t *__restrict__ counts)
+{
+    const uint64_t id = global_id();
+    if (id >= numGroups * 16u) return;
+    atomicAdd(&counts[recs[(id >> 4) * CUTE_QUAD_RECORD_WORDS + (id & 15u)]], 1u);
+}
+
+__global__ __launch_bounds__(kThreads) void mark_hub_columns(const uint32_t *__restrict__ recs, uint64_t numGroups,
+                                                             const uint32_t *__restrict__ slot_of, uint32_t hub_flag,
+                                                             uint32_t *__restrict__ out)
+{
+    const uint64_t id = global_id();
+    if (id >= numGroups * CUTE_QUAD_RECORD_WORDS) return;
+    uint32_t w = recs[id];
+    if (id % CUTE_QUAD_RECORD_WORDS < 16u) {
+        const uint32_t slot = slot_of[w];
+        if (slot != ~0u) w = hub_flag | slot;
+    }
+    out[id] = w;
+}
+
 }  // namespace cute_build

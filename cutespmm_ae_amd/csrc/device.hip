@@ -19,7 +19,8 @@ thread_local std::string g_hip_error;
 // The planner's default thresholds (measured on the five benchmark matrices and on the reference's 43).
 constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
 constexpr float kWideReuse = 0.98f;          // ... the bar for products of 256 columns or more over large matrices (see cute_spmm_plan_create)
-constexpr uint32_t kMaxRowForRows = 48;     // ... unless it holds a row longer than this: one lane group would serialise it
+constexpr uint32_t kMaxRowForRows = 48;
+constexpr uint32_t kMaxHubRows = 256;       // hub plans: B rows a work-group keeps in LDS (64 KiB of 256-byte pieces; two work-groups per CU)     // ... unless it holds a row longer than this: one lane group would serialise it
 constexpr float kHybridFill = 0.15f;         // cute_hybrid: a tile goes to the Blocked-ELL part from this fill on (threshold 0)
 constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
 // B and C together larger than the Infinity Cache: whatever the caller does between launches, their rows come
@@ -193,6 +194,10 @@ struct cute_spmm_plan {
     uint32_t rows_slabs = 1;
     uint4 *dChunks = nullptr;
     uint32_t *dHeads = nullptr;         // quad kernels: per chunk, the descriptor and the record of its first group
+    // hub plans: the most referenced B rows are staged in LDS by persistent work-groups (hrpb_quad_hub_f32)
+    uint32_t numHub = 0;
+    uint32_t *dHubRows = nullptr;       // the hub rows' column ids, slot order
+    uint32_t *dHubRecs = nullptr;       // the plan's copy of the quad records, hub columns replaced by their slots
     // panels (or 4-row strips) cut into several chunks: each chunk stores a partial tile, reduce_partials adds them
     uint4 *dFixups = nullptr;           // {panel or strip, first piece, pieces, -}
     uint32_t numFixups = 0;
@@ -594,6 +599,41 @@ int finish_upload(cute_hrpb_dev *d, const uint32_t *rowPtr, int quad_layout, con
     return rc;
 }
 
+// Tables of a hub plan: the hub_rows most referenced columns of the quad records (ties: the lower column) get
+// the slots 0.. of the LDS table; the plan keeps their column ids in slot order and its own copy of the records
+// in which those columns name their slot.
+int make_hub_tables(cute_spmm_plan *p, const cute_hrpb_dev *d, uint32_t hub_rows)
+{
+    const uint64_t G = d->numGroups;
+    DevBuf counts, slots;
+    int rc = counts.alloc(uint64_t(d->K) * 4u);
+    if (rc == CUTE_OK) rc = slots.alloc(uint64_t(d->K) * 4u);
+    if (rc != CUTE_OK) return rc;
+    HIP_TRY(hipMemset(counts.p, 0, uint64_t(d->K) * 4u));
+    hipLaunchKernelGGL(cute_build::count_record_columns, grid_of(G * 16u), dim3(cute_build::kThreads), 0, nullptr, d->dQRecs, G,
+                       counts.as<uint32_t>());
+    std::vector<uint32_t> cnt(d->K), order(d->K), slot_of(d->K, ~0u);
+    HIP_TRY(hipMemcpy(cnt.data(), counts.p, uint64_t(d->K) * 4u, hipMemcpyDeviceToHost));
+    for (uint32_t k = 0; k < d->K; ++k) order[k] = k;
+    std::partial_sort(order.begin(), order.begin() + hub_rows, order.end(),
+                      [&](uint32_t a, uint32_t b) { return cnt[a] != cnt[b] ? cnt[a] > cnt[b] : a < b; });
+    uint32_t used = 0;
+    while (used < hub_rows && cnt[order[used]] > 1u) ++used;            // a row fetched once gains nothing from LDS
+    if (!used) return CUTE_OK;
+    for (uint32_t h = 0; h < used; ++h) slot_of[order[h]] = h;
+    HIP_TRY(hipMemcpy(slots.p, slot_of.data(), uint64_t(d->K) * 4u, hipMemcpyHostToDevice));
+    rc = upload(&p->dHubRows, order.data(), used);
+    if (rc != CUTE_OK) return rc;
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&p->dHubRecs), std::max<uint64_t>(G * CUTE_QUAD_RECORD_WORDS * 4u, 16u)));
+    hipLaunchKernelGGL(cute_build::mark_hub_columns, grid_of(G * CUTE_QUAD_RECORD_WORDS), dim3(cute_build::kThreads), 0, nullptr,
+                       d->dQRecs, G, slots.as<const uint32_t>(), uint32_t(cute_dev::kHubFlag), p->dHubRecs);
+    rc = check_launch("hub records");
+    if (rc != CUTE_OK) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    p->numHub = used;
+    return CUTE_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -705,6 +745,8 @@ void cute_spmm_plan_free(cute_spmm_plan *p)
     if (!p) return;
     (void)hipFree(p->dChunks);
     (void)hipFree(p->dHeads);
+    (void)hipFree(p->dHubRows);
+    (void)hipFree(p->dHubRecs);
     (void)hipFree(p->dFixups);
     (void)hipFree(p->dPartials);
     (void)hipFree(p->dRowList);
@@ -961,8 +1003,17 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     // the mean), or the eighths of the list differ by more than a tenth in work, the long items go first and the list
     // is dealt round-robin to the XCDs: items are ordered by the power of two of their length only, so neighbours of
     // similar length stay neighbours and keep sharing B rows in the L2.
-    bool longest_first = t.chunk_order == 3;
-    if (t.chunk_order == 0 && !chunks.empty()) {
+    // Hub plans: the strips of a graph with hub vertices through persistent work-groups that keep the most
+    // referenced B rows in LDS.  Opt-in (cute_tunables.hub_rows); needs the quad kernel on strip lists.
+    const uint32_t hub_rows = (t.hub_rows && p->shape == 2 && d->quadRows == 4 && !chunks.empty())
+                                  ? std::min<uint32_t>(std::min<uint32_t>(t.hub_rows, kMaxHubRows), d->K) : 0u;
+    if (hub_rows) {
+        // work items are dealt to the wavefronts of the resident work-groups in list order: longest first
+        std::stable_sort(chunks.begin(), chunks.end(), [](const uint4 &a, const uint4 &b) { return a.y - a.x > b.y - b.x; });
+        p->info.dealtChunks = 2;
+    }
+    bool longest_first = t.chunk_order == 3 && !hub_rows;
+    if (t.chunk_order == 0 && !chunks.empty() && !hub_rows) {
         const uint64_t resident = uint64_t(c.num_cus) * 4u * ((p->shape == 2 || p->ng == 1) ? 8u : 4u);
         uint64_t total = 0;
         uint32_t longest = 0;
@@ -1009,12 +1060,13 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         }
         p->info.dealtChunks = 2;
     } else
-    if (t.chunk_order != 1 && c.whole_chip && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
+    if (t.chunk_order != 1 && !hub_rows && c.whole_chip && (p->shape == 2 || p->pipeline == 1) && !chunks.empty())
         p->info.dealtChunks = deal_chunks(chunks, num_slabs, uint32_t(c.num_cus) / cute_dev::kNumXcd,
                                           p->shape == 2 || p->ng == 1 ? 8u : 4u, t.chunk_order == 2) ? 1u : 0u;
     // the layout this plan's MFMA kernel reads, if the upload has not built it
     int rc = chunks.empty() ? int(CUTE_OK) : ensure_layout(d, p->shape);
     if (rc == CUTE_OK) rc = upload(&p->dChunks, chunks.data(), chunks.size());
+    if (rc == CUTE_OK && hub_rows) rc = make_hub_tables(p, d, hub_rows);
     if (rc == CUTE_OK && p->shape == 2 && !chunks.empty()) {
         // one 128-byte head per work item: its descriptor and a copy of its first group's record, so that a
         // wavefront can ask for its first B rows after one scalar fetch instead of two dependent ones; gathered
@@ -1023,7 +1075,7 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         if (hipMalloc(reinterpret_cast<void **>(&p->dHeads), words * sizeof(uint32_t)) != hipSuccess) rc = CUTE_ERR_NOMEM;
         if (rc == CUTE_OK) {
             hipLaunchKernelGGL(cute_build::quad_heads, grid_of(words), dim3(cute_build::kThreads), 0, nullptr, p->dChunks,
-                               uint32_t(chunks.size()), d->dQRecs, uint32_t(cute_dev::kQuadHeadWords), p->dHeads);
+                               uint32_t(chunks.size()), p->dHubRecs ? p->dHubRecs : d->dQRecs, uint32_t(cute_dev::kQuadHeadWords), p->dHeads);
             rc = check_launch("quad heads");
             if (rc == CUTE_OK && hipStreamSynchronize(nullptr) != hipSuccess) rc = CUTE_ERR_HIP;
         }
@@ -1059,13 +1111,14 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     p->info.precision = p->bf16x3 ? uint32_t(CUTE_PREC_BF16X3) : uint32_t(CUTE_PREC_FP32);
     p->info.path = uint32_t(t.path);
     p->info.mfmaShape = uint32_t(p->shape);
+    p->info.hubRows = p->numHub;
     p->info.pipeline = uint32_t(p->pipeline);
     // one launch for a mixed plan: the quad kernel with any row shape of 4-float lanes, the rolling brick
     // kernel in the shapes the planner itself picks for N (forced column groups fall back to two launches)
     const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
     const bool brick_default_shape = ng_for_mixed || p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
     p->info.partialTileKiB = uint32_t((p->partialBytes + 1023u) / 1024u);
-    p->info.fusedLaunch = (rows_fusable && !p->bf16x3 && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
+    p->info.fusedLaunch = (rows_fusable && !p->bf16x3 && !p->numHub && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
     *out = p;
     return CUTE_OK;
 }
@@ -1274,7 +1327,18 @@ int run_with(const cute_spmm_plan *p, const float *dB, float *dC, void *stream, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t N = p->info.N;
     bool rows_launched = false;        // the sparse rows went out together with the MFMA chunks
-    if (p->info.numChunks && p->shape == 2) {
+    if (p->info.numChunks && p->shape == 2 && p->numHub) {
+        // persistent work-groups of sixteen wavefronts, two per compute unit, each with the hub rows of its slab in LDS
+        const uint32_t wgs = std::min<uint32_t>(2u * uint32_t(context().num_cus), (p->info.numChunks + cute_dev::kHubWaves - 1) / cute_dev::kHubWaves);
+        const dim3 grid(wgs, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kHubWaves);
+        const size_t lds = size_t(p->numHub) * cute_dev::kWaveSize * sizeof(float);
+        if (N % 64u == 0)
+            hipLaunchKernelGGL((cute_dev::hrpb_quad_hub_f32<true>), grid, block, lds, s, p->dHeads, p->info.numChunks, p->dHubRecs,
+                               p->d->dQVals, uint32_t(p->d->numQuadVals), p->dHubRows, p->numHub, dB, dC, partials, N);
+        else
+            hipLaunchKernelGGL((cute_dev::hrpb_quad_hub_f32<false>), grid, block, lds, s, p->dHeads, p->info.numChunks, p->dHubRecs,
+                               p->d->dQVals, uint32_t(p->d->numQuadVals), p->dHubRows, p->numHub, dB, dC, partials, N);
+    } else if (p->info.numChunks && p->shape == 2) {
         const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
         const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);

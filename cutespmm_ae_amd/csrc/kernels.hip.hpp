@@ -565,10 +565,24 @@ __device__ __forceinline__ void quad_mfma(float a, float b, f32x4 (&acc)[4])
     acc[P & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, acc[P & 3], 4, P, 0);
 }
 
-__device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32_t col, uint32_t row_pitch, uint32_t col_off)
+// HUB: the column words of the records a hub plan reads may name a slot of the work-group's LDS table of hub
+// rows instead of a B row (kHubFlag | slot): that operand then comes out of LDS (see hrpb_quad_hub_f32).
+constexpr uint32_t kHubFlag = 0x80000000u;
+
+template <bool HUB>
+__device__ __forceinline__ float quad_load_b(const float *__restrict__ B, uint32_t col, uint32_t row_pitch, uint32_t col_off,
+                                             const float *hub)
 {
+    if (HUB && (col & kHubFlag))        // wave-uniform: the column is a scalar
+        return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(hub) + ((col & 0x00ffffffu) * (kWaveSize * 4u) + (threadIdx.x & (kWaveSize - 1)) * 4u));
     return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(B) + (__umul24(col, row_pitch) + col_off));
 }
+
+template <bool FULL, bool STRIPS, bool HUB>
+__device__ __forceinline__ void quad_chunk(uint32_t chunk, uint32_t block_y, const uint32_t *__restrict__ heads,
+                                           const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
+                                           const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials,
+                                           uint32_t N, const float *hub);
 
 template <bool FULL, bool STRIPS>
 __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, const uint32_t *__restrict__ heads,
@@ -577,10 +591,19 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
                                           const float *__restrict__ B, float *__restrict__ C,
                                           float *__restrict__ partials, uint32_t N)
 {
-    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
     const uint32_t chunk = xcd_contiguous_id(block_x, groups_per_xcd) * kWavesPerGroup + wave;
     if (chunk >= num_chunks) return;
+    quad_chunk<FULL, STRIPS, false>(chunk, block_y, heads, qrecs, qvals, zero_index, B, C, partials, N, nullptr);
+}
+
+template <bool FULL, bool STRIPS, bool HUB>
+__device__ __forceinline__ void quad_chunk(uint32_t chunk, uint32_t block_y, const uint32_t *__restrict__ heads,
+                                           const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
+                                           const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials,
+                                           uint32_t N, const float *hub)
+{
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     // One entry of kQuadHeadWords per chunk: its descriptor and, behind it, the record of its first group, so
     // that the first B rows can be requested after one scalar fetch instead of two dependent ones.
     const uint32_t *head = heads + size_t(chunk) * kQuadHeadWords;
@@ -630,13 +653,13 @@ __device__ __forceinline__ void quad_body(uint32_t block_x, uint32_t block_y, co
         a0 = fetch_a(ca);
         a1 = fetch_a(cb);
 #pragma unroll
-        for (int p = 0; p < 16; ++p) b0[p] = quad_load_b(B, ca[p], row_pitch, col_off);
+        for (int p = 0; p < 16; ++p) b0[p] = quad_load_b<HUB>(B, ca[p], row_pitch, col_off, hub);
 #pragma unroll
-        for (int p = 0; p < 16; ++p) b1[p] = quad_load_b(B, cb[p], row_pitch, col_off);
+        for (int p = 0; p < 16; ++p) b1[p] = quad_load_b<HUB>(B, cb[p], row_pitch, col_off, hub);
 #define CUTE_QUAD_ROLL(P, A, BSET, COLS)                          \
     quad_mfma<P>(A, BSET[P], acc);                                \
     __builtin_amdgcn_sched_barrier(0);                            \
-    BSET[P] = quad_load_b(B, COLS[P], row_pitch, col_off);        \
+    BSET[P] = quad_load_b<HUB>(B, COLS[P], row_pitch, col_off, hub); \
     __builtin_amdgcn_sched_barrier(0);
 #define CUTE_QUAD_ROLL_REST(A, BSET, COLS)                                                                 \
     CUTE_QUAD_ROLL(1, A, BSET, COLS) CUTE_QUAD_ROLL(2, A, BSET, COLS)                                      \
@@ -716,6 +739,36 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_f32(
 {
     quad_body<FULL, STRIPS>(blockIdx.x, blockIdx.y, heads, num_chunks, groups_per_xcd, qrecs, qvals, zero_index, B, C,
                             partials, N);
+}
+
+// ---------------------------------------------------------------------------------------
+// The quad kernel with the most referenced B rows staged in LDS (the reference stages the B rows of a block in
+// shared memory for the warps of its thread block, kernel.cu:123-124,143-164; here what is staged is what many
+// work items share: the rows of hub columns).  A work-group of sixteen wavefronts copies, once, the 64-column
+// pieces of `num_hub` hub rows of its slab into LDS (num_hub * 256 bytes) and then stays: its wavefronts walk the
+// chunk list with a stride of the whole launch, so the table is filled once per work-group, not once per chunk.
+// A column word of the plan's records that carries kHubFlag names a slot of that table, and the operand is an
+// LDS read instead of a gather through the vector memory path.  Strip lists only (graphs with hub vertices).
+// ---------------------------------------------------------------------------------------
+constexpr int kHubWaves = 16;
+
+template <bool FULL>
+__global__ __launch_bounds__(kWaveSize *kHubWaves) void hrpb_quad_hub_f32(
+    const uint32_t *__restrict__ heads, uint32_t num_chunks, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals,
+    uint32_t zero_index, const uint32_t *__restrict__ hub_rows, uint32_t num_hub, const float *__restrict__ B,
+    float *__restrict__ C, float *__restrict__ partials, uint32_t N)
+{
+    extern __shared__ float hub[];
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const uint32_t n = blockIdx.y * kWaveSize + lane;
+    for (uint32_t h = wave; h < num_hub; h += kHubWaves)
+        hub[h * kWaveSize + lane] = (FULL || n < N) ? B[size_t(hub_rows[h]) * N + n] : 0.0f;
+    __syncthreads();
+    // consecutive chunks of the list (longest first) go to different work-groups
+    const uint32_t stride = gridDim.x * kHubWaves;
+    for (uint32_t chunk = wave * gridDim.x + blockIdx.x; chunk < num_chunks; chunk += stride)
+        quad_chunk<FULL, true, true>(chunk, blockIdx.y, heads, qrecs, qvals, zero_index, B, C, partials, N, hub);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -436,7 +436,9 @@ typedef struct cute_tunables {
                                   cache holds); 2 cache-resident (a tight loop over the same operands that fit the 256 MiB
                                   Infinity Cache together; ignored when they do not).  Chooses between the MFMA kernels
                                   (and, for 1, keeps two column groups per lane in mixed plans), nothing else. */
-    uint32_t reserved[1];
+    uint32_t hub_rows;         /* > 0 (at most 256): the quad kernel on strip lists runs as persistent work-groups that keep that many
+                                  of the most referenced B rows in LDS (graphs with hub vertices); 0: off.  Ignored by other plans
+                                  (cute_plan_info.hubRows says how many rows a plan stages) */
 } cute_tunables;
 
 typedef struct cute_plan_info {
@@ -453,6 +455,7 @@ typedef struct cute_plan_info {
     uint32_t fusedLaunch;      /* 1: MFMA chunks and sparse rows go out as one launch     */
     uint32_t dealtChunks;      /* 1: the MFMA work items were dealt to the SIMDs by length, 2: listed long items first, 0: panel order (cute_tunables.chunk_order) */
     uint32_t partialTileKiB;   /* KiB of partial tiles the pieces of cut panels store per launch (0: no panel is cut) */
+    uint32_t hubRows;          /* B rows a hub plan keeps in LDS (0: not a hub plan) */
 } cute_plan_info;
 
 typedef struct cute_spmm_plan cute_spmm_plan;

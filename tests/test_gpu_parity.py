@@ -450,6 +450,47 @@ def test_wide_products_of_short_rows_go_to_the_quad_kernel(cs, orc, torch_cuda):
     assert cs.SPMM_TC(h, 512, min_reuse=1.25).info["numChunks"] == 0
 
 
+def test_hub_rows_staged_in_lds(cs, orc, torch_cuda):
+    """cute_tunables.hub_rows: the quad kernel on strip lists as persistent work-groups with the most referenced B
+    rows in LDS.  A graph-like matrix (a few columns in most rows, a few very long rows): exact on integers, within
+    tolerance on real values, widths that are and are not multiples of the 64-column slab, cut strips included."""
+    torch = torch_cuda
+    rng = np.random.default_rng(31)
+    M, K = 2048, 6000 // 16 * 16
+    hubs = rng.choice(K, 40, replace=False)
+
+    def row(r):
+        n = 1500 if r in (9, 700, 701) else 4
+        mine = set(int(x) for x in rng.choice(K, n, replace=False))
+        mine.update(int(x) for x in hubs[rng.random(40) < 0.5])
+        return sorted(mine)
+    lists = [row(r) for r in range(M)]
+    rp = np.concatenate([[0], np.cumsum([len(x) for x in lists])]).astype(np.uint32)
+    cl = np.concatenate(lists).astype(np.uint32)
+    for values, exact in (("ints", True), ("normal", False)):
+        vl = rng.integers(-4, 5, len(cl)).astype(np.float32) if exact else rng.standard_normal(len(cl)).astype(np.float32)
+        h = cs.HRPB(M, K, rp, cl, vl)
+        assert h.upload(quad_layout=2)
+        for N in (64, 128, 200):
+            B = (rng.integers(-3, 4, (K, N)) if exact else rng.standard_normal((K, N))).astype(np.float32)
+            ref = orc.spmm_csr(rp, cl, vl, B)
+            for hub_rows in (256, 16, 1000):
+                out, plan = _run(cs, torch, h, B, path=cs.PATH_BRICK, mfma_shape=2, hub_rows=hub_rows)
+                assert plan.kernel_name == "hrpb_quad_hub_f32" and 0 < plan.info["hubRows"] <= min(hub_rows, 256), plan.info
+                assert plan.info["numAtomicChunks"] > 0
+                if exact:
+                    assert (out == ref).all(), (N, hub_rows)
+                else:
+                    assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (N, hub_rows)
+            # mixed with the row kernel (the planner's own split) and as the plain quad kernel: the same product
+            out, plan = _run(cs, torch, h, B, hub_rows=128)
+            assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
+    # plans that are not the quad kernel on strip lists ignore the tunable
+    A = cs.gen_config(2, 1 / 16.0)
+    h2 = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    assert cs.SPMM_TC(h2, 128, hub_rows=256).info["hubRows"] == 0
+
+
 def test_layouts_are_built_when_first_needed(cs, orc, torch_cuda):
     """An upload sends the CSR arrays and the one MFMA layout the planner's default rules would use (none when every
     panel would go to the row kernel); a plan that asks for the other one builds it then, from the device copy of the

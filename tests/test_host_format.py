@@ -39,7 +39,7 @@ def test_struct_sizes_match_header(cs):
     assert C.sizeof(cs.cute_hrpb_host) == 88
     assert C.sizeof(cs.cute_hrpb_tiled) == 48
     assert C.sizeof(cs.cute_tunables) == 48
-    assert C.sizeof(cs.cute_plan_info) == 64
+    assert C.sizeof(cs.cute_plan_info) == 68
 
 
 def test_status_strings(cs):
