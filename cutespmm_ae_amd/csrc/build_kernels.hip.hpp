@@ -153,14 +153,22 @@ __global__ __launch_bounds__(kThreads) void entry_positions(const uint32_t *__re
 }
 
 // Active columns per panel and list pairs per strip, from the prefix sums DP, DS of the first-of-column flags.
-__global__ __launch_bounds__(kThreads) void count_columns(const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ DP,
-                                                          const uint32_t *__restrict__ DS, uint32_t P,
-                                                          uint32_t *__restrict__ panelCols, uint32_t *__restrict__ stripPairs)
+// Also the width of every panel's column window (last column - first column + 1; rows are sorted).
+__global__ __launch_bounds__(kThreads) void count_columns(const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols,
+                                                          const uint32_t *__restrict__ DP, const uint32_t *__restrict__ DS,
+                                                          uint32_t P, uint32_t *__restrict__ panelCols,
+                                                          uint32_t *__restrict__ stripPairs, uint32_t *__restrict__ panelSpan)
 {
     const uint64_t id = global_id();
     if (id < P) {
         const uint32_t s = rowPtr[id * 16u], e = rowPtr[id * 16u + 16u];
         panelCols[id] = e > s ? DP[e - 1u] - DP[s] + 1u : 0u;
+        uint32_t lo = ~0u, hi = 0u;
+        for (uint32_t r = 0; r < 16u; ++r) {
+            const uint32_t rs = rowPtr[id * 16u + r], re = rowPtr[id * 16u + r + 1u];
+            if (re > rs) { lo = min(lo, cols[rs]); hi = max(hi, cols[re - 1u]); }
+        }
+        panelSpan[id] = e > s ? hi - lo + 1u : 0u;
     }
     if (id < uint64_t(P) * 4u) {
         const uint32_t s = rowPtr[id * 4u], e = rowPtr[id * 4u + 4u];

@@ -18,6 +18,7 @@ thread_local std::string g_hip_error;
 
 // The planner's default thresholds (measured on the five benchmark matrices and on the reference's 43).
 constexpr float kMinReuse = 1.25f;          // a panel with fewer nonzeros per B row the MFMA side would fetch goes to the row kernel
+constexpr uint64_t kWideWindowBytes = 16ull << 20;   // ... whose window of B is wider than this (four L2s' worth)
 constexpr float kWideReuse = 0.98f;          // ... the bar for products of 256 columns or more over large matrices (see cute_spmm_plan_create)
 constexpr uint32_t kMaxRowForRows = 48;
 constexpr uint32_t kMaxHubRows = 256;       // hub plans: B rows a work-group keeps in LDS (64 KiB of 256-byte pieces; two work-groups per CU)     // ... unless it holds a row longer than this: one lane group would serialise it
@@ -181,6 +182,7 @@ struct cute_hrpb_dev {
     std::vector<uint32_t> panelNnz;     // nonzeros per row panel
     std::vector<uint32_t> panelCols;    // active columns per row panel
     std::vector<uint32_t> panelMaxRow;  // longest row of each panel
+    std::vector<uint32_t> panelSpan;    // width of each panel's column window (last column - first column + 1)
 };
 
 struct cute_spmm_plan {
@@ -377,11 +379,13 @@ struct Census {
     DevBuf rowOf, posP, posS, DP, DS;
 };
 
-int device_census(const cute_hrpb_dev *d, Census &c, std::vector<uint32_t> *panelCols, std::vector<uint32_t> *stripPairs)
+int device_census(const cute_hrpb_dev *d, Census &c, std::vector<uint32_t> *panelCols, std::vector<uint32_t> *stripPairs,
+                  std::vector<uint32_t> *panelSpan = nullptr)
 {
     const uint32_t nnz = d->nnz, P = d->P;
     if (panelCols) panelCols->assign(P, 0u);
     if (stripPairs) stripPairs->assign(size_t(P) * 4u, 0u);
+    if (panelSpan) panelSpan->assign(P, 0u);
     if (!nnz) return CUTE_OK;
     const uint64_t bytes = uint64_t(nnz) * sizeof(uint32_t);
     int rc = c.rowOf.alloc(bytes);
@@ -406,14 +410,16 @@ int device_census(const cute_hrpb_dev *d, Census &c, std::vector<uint32_t> *pane
     if (rc == CUTE_OK) rc = device_scan(c.DP.as<uint32_t>(), nnz);
     if (rc == CUTE_OK) rc = device_scan(c.DS.as<uint32_t>(), nnz);
     if (rc != CUTE_OK || !panelCols || !stripPairs) return rc;
-    DevBuf pc, sp;
+    DevBuf pc, sp, span;
     rc = pc.alloc(uint64_t(P) * 4u);
     if (rc == CUTE_OK) rc = sp.alloc(uint64_t(P) * 16u);
+    if (rc == CUTE_OK) rc = span.alloc(uint64_t(P) * 4u);
     if (rc != CUTE_OK) return rc;
-    hipLaunchKernelGGL(cute_build::count_columns, grid_of(uint64_t(P) * 4u), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr,
-                       c.DP.as<const uint32_t>(), c.DS.as<const uint32_t>(), P, pc.as<uint32_t>(), sp.as<uint32_t>());
+    hipLaunchKernelGGL(cute_build::count_columns, grid_of(uint64_t(P) * 4u), dim3(cute_build::kThreads), 0, nullptr, d->dRowPtr, d->dCols,
+                       c.DP.as<const uint32_t>(), c.DS.as<const uint32_t>(), P, pc.as<uint32_t>(), sp.as<uint32_t>(), span.as<uint32_t>());
     HIP_TRY(hipMemcpy(panelCols->data(), pc.p, uint64_t(P) * 4u, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(stripPairs->data(), sp.p, uint64_t(P) * 16u, hipMemcpyDeviceToHost));
+    if (panelSpan) HIP_TRY(hipMemcpy(panelSpan->data(), span.p, uint64_t(P) * 4u, hipMemcpyDeviceToHost));
     return CUTE_OK;
 }
 
@@ -575,7 +581,7 @@ int finish_upload(cute_hrpb_dev *d, const uint32_t *rowPtr, int quad_layout, con
 {
     Census cen;
     std::vector<uint32_t> strip_pairs;
-    int rc = device_census(d, cen, &d->panelCols, &strip_pairs);
+    int rc = device_census(d, cen, &d->panelCols, &strip_pairs, &d->panelSpan);
     if (rc != CUTE_OK) return rc;
     d->brp.assign(size_t(d->P) + 1, 0u);
     d->panelNnz.resize(d->P);
@@ -779,7 +785,7 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     const uint32_t max_row_for_rows = t.max_row_nnz ? t.max_row_nnz : kMaxRowForRows;
     // An MFMA work item always spans 64 output columns; when N is narrower the row kernel wastes
     // less, so the reuse a panel must offer to earn the MFMA kernel grows (measured on N = 8..32).
-    float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
+    const float reuse_bar = N <= 32 ? std::min(3.0f, min_reuse * 48.0f / float(N)) : min_reuse;
     // Wide products of large matrices: the row kernel walks three dependent round trips per row (row pointers,
     // entries, B rows), the quad kernel streams its lists two groups ahead, and with 256 columns or more and a launch
     // several times the size of the device that depth counts for more than reuse: on 50 000 rows of 7 entries at
@@ -787,8 +793,11 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     // reference's matrices gain 10-20 % the same way.  There the bar drops to "the lists need no more fetches than the
     // panel has entries" (matrices whose short lists would be mostly padding -- cat_ears_4_4, Wordnet3 -- stay with
     // the row kernel, which is 20 % ahead on them).
-    if (t.min_reuse <= 0.0f && N >= 256u && uint64_t(d->M) * ((N + 255u) / 256u) >= 4ull * uint64_t(c.num_cus) * 32u)
-        reuse_bar = kWideReuse;
+    // ... provided the panel's B rows cannot come out of an L2 anyway: a banded matrix, whose panels read a window of B
+    // that the L2s hold (the banded benchmark matrix: 4 112 columns), is bound by the L2-to-L1 gather rate, where the row
+    // kernel's 16 bytes per lane beat the quad kernel's 4 (1 736 against 2 046 us), and keeps the usual bar.
+    const bool wide_and_large = t.min_reuse <= 0.0f && N >= 256u &&
+                                uint64_t(d->M) * ((N + 255u) / 256u) >= 4ull * uint64_t(c.num_cus) * 32u;
 
     cute_spmm_plan *p = new cute_spmm_plan;
     p->d = d;
@@ -809,7 +818,8 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
             // lists (pairs plus padding), which is at least one per active column
             const uint32_t lists = d->quadRows == 4 ? 4u : 1u;
             const uint32_t fetches = std::max(d->panelCols[q], (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u);
-            rows = float(d->panelNnz[q]) < reuse_bar * float(fetches) && d->panelMaxRow[q] <= max_row_for_rows;
+            const float bar = (wide_and_large && uint64_t(d->panelSpan[q]) * N * sizeof(float) > kWideWindowBytes) ? kWideReuse : reuse_bar;
+            rows = float(d->panelNnz[q]) < bar * float(fetches) && d->panelMaxRow[q] <= max_row_for_rows;
         }
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;

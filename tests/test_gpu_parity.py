@@ -412,6 +412,10 @@ def test_default_kernel_choice(cs, orc, torch_cuda):
     assert cs.SPMM_TC(h, 128, operand_residency=1).kernel_name == "hrpb_brick_f32_rolling"
     assert cs.SPMM_TC(h, 128, operand_residency=2).kernel_name == "hrpb_quad_f32"
     assert cs.SPMM_TC(h, 1024, operand_residency=2).kernel_name == "hrpb_brick_f32_rolling"   # 512 MiB: no cache holds that
+    # the banded benchmark matrix (an eighth of it) at its own width: wide and large, but its panels read a window of B the
+    # L2s hold, so the rule for wide products of short rows leaves it with the row kernel
+    A5 = cs.gen_config(5, 1 / 8.0)
+    assert cs.SPMM_TC(cs.HRPB(A5.M, A5.K, A5.rowPtr, A5.cols, A5.vals), 256).kernel_name == "csr_rows_batched"
     M, rp, cl, vl = _stencil5(200)
     h5 = cs.HRPB(M, M, rp, cl, vl)
     B = np.random.default_rng(5).standard_normal((M, 128)).astype(np.float32)
