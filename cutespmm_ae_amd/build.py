@@ -9,6 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libcutespmm.so")
 DRIVER = os.path.join(HERE, "run_cute")
+PROBE = os.path.join(HERE, "membw_probe")
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
@@ -58,9 +59,17 @@ def build_driver():
     return DRIVER
 
 
+def build_probe():
+    """The memory-pattern microbenchmark (a stand-alone HIP program; nothing of the library links to it)."""
+    src = os.path.join(CSRC, "membw_probe.hip")
+    _run([HIPCC, "-x", "hip", src, "-o", PROBE] + COMMON + DEVICE_FLAGS)
+    return PROBE
+
+
 def build_all():
     build_library()
     build_driver()
+    build_probe()
 
 
 if __name__ == "__main__":
