@@ -193,6 +193,26 @@ def other_config(torch, cs, config, stream, precision=None):
     return res
 
 
+def memory_pattern_probe():
+    """Runs cutespmm_ae_amd/membw_probe (plain streaming kernels, no SpMM) as a child process and returns its
+    HBM-fed ("rotating") times in microseconds, keyed by pattern; None if the program is not built or fails.
+    Called before this process touches the GPU."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cutespmm_ae_amd", "membw_probe")
+    if not os.path.exists(exe):
+        return None
+    try:
+        text = subprocess.run([exe], capture_output=True, text=True, timeout=120, check=True).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    out = {}
+    for line in text.splitlines():
+        parts = line.rsplit("rotating", 1)
+        if len(parts) == 2 and " us" in parts[1]:
+            out[" ".join(parts[0].split())] = float(parts[1].split("us")[0])
+    return out or None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -222,11 +242,19 @@ def main():
                     help="MFMA work items: 0 planner's choice, 1 panel order, 2 dealt to the SIMDs longest first")
     ap.add_argument("--graph", action="store_true",
                     help="record the K launches of the timed region into one HIP graph and replay it (launch-bound workloads; one buffer set)")
+    ap.add_argument("--no-probe", action="store_true", help="skip the memory-pattern microbenchmark (hbm_fed.plain_streaming_kernels_us)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run 10 plain device copies of 32 MiB and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (got --gpus %d); nothing here shards across GPUs" % args.gpus)
+
+    # plain streaming kernels of the headline's size for scale; a child process, started before this one uses the GPU
+    # (not under a profiler: its preloaded library would profile the child as well)
+    profiled = any("rocprof" in v.lower() for v in (os.environ.get("LD_PRELOAD", ""), os.environ.get("ROCP_TOOL_LIBRARIES", "")))
+    probe = None
+    if args.config == 2 and not (args.no_probe or args.calibrate_copy or args.graph or args.no_resident_leg or profiled):
+        probe = memory_pattern_probe()
 
     import torch
     import cutespmm_ae_amd as cs
@@ -344,6 +372,10 @@ def main():
                                              for name, shape in (("quad", 2), ("brick", 1))}
             fed["device_copy_of_B_onto_C_us"] = timed_steps(torch, type("Copy", (), {"run": staticmethod(lambda b, c: c.copy_(b))}), dBs, dCs,
                                                             steps2, 50, 0.0, stream)[1] * 1e3
+        if probe:
+            fed["plain_streaming_kernels_us"] = dict(
+                note="cutespmm_ae_amd/membw_probe: 4 096 wavefronts that stream private regions, rotating buffer sets (HBM-fed); "
+                     "for scale against this launch's bytes beyond the L2s (roofline.traffic)", **probe)
         out["hbm_fed"] = fed
     plan.run(dB, dC)
     torch.cuda.synchronize()
