@@ -84,3 +84,42 @@ def test_random_plans_equal_the_oracle(cs, orc, torch_cuda, kind):
             assert np.array_equal(dC.cpu().numpy(), ref), what + " -> " + p.kernel_name
             launches += 1
     assert launches == 40
+
+
+def test_random_special_paths_equal_the_oracle(cs, orc, torch_cuda):
+    """The same on the paths a default plan never takes: the bf16x3 brick kernel (small integers split into an exact
+    high part and a zero low part), the hub kernel on strip lists, the hybrid call under both split rules, and the
+    three plain CSR kernels."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77001)
+    for case in range(14):
+        kind = KINDS[case % len(KINDS)]
+        M, K, rp, cl, vl = _matrix(rng, kind)
+        N = int(rng.choice(WIDTHS[:-1]))
+        if M * N > (1 << 20):
+            N = max(1, (1 << 20) // M)
+        B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        dB = torch.from_numpy(B).cuda()
+        h = cs.HRPB(M, K, rp, cl, vl)
+        strips = cs.DeviceHRPB(M, K, torch.from_numpy(rp.astype(np.int64).astype(np.int32)).cuda(),
+                               torch.from_numpy(cl.view(np.int32).copy()).cuda(), torch.from_numpy(vl.copy()).cuda(), quad_layout=2)
+        for handle, kw in ((h, dict(precision=cs.PREC_BF16X3)), (h, dict(precision=cs.PREC_BF16X3, slots=3, max_chunk_blocks=1)),
+                           (strips, dict(path=cs.PATH_BRICK, mfma_shape=2, hub_rows=int(rng.choice([1, 8, 64, 256]))))):
+            p = cs.SPMM_TC(handle, N, **kw)
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            p.run(dB, dC)
+            torch.cuda.synchronize()
+            assert np.array_equal(dC.cpu().numpy(), ref), (kind, case, M, K, N, kw, p.kernel_name)
+        csr = cs.CSR_Matrix(nrows=M, ncols=K, rowPtr=rp.astype(np.int32), cols=cl.astype(np.int32), values=vl)
+        for kw in (dict(), dict(nnz_threshold=int(rng.integers(1, 60))),
+                   dict(mode=cs.HYBRID_CLASSIFIER, deviation_threshold=float(rng.random()), underload_dominance=float(rng.random()))):
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            cs.HybridSpMM(csr, **kw).spmm(dB, dC)
+            torch.cuda.synchronize()
+            assert np.array_equal(dC.cpu().numpy(), ref), (kind, case, M, K, N, kw)
+        for alg in (0, 1, 2):
+            dC = torch.full((M, N), float("nan"), device="cuda")
+            cs.csr_spmm_dev(alg, h, dB, dC)
+            torch.cuda.synchronize()
+            assert np.array_equal(dC.cpu().numpy(), ref), (kind, case, M, K, N, "csr kernel", alg)
