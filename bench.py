@@ -53,8 +53,11 @@ def recorded_traffic(workload, kernel):
     rel = "profiles/hbm_traffic_%s.json" % workload
     try:
         rec = json.load(open(os.path.join(ROOT, rel))).get(workload)
+        for name, other in (rec.get("other_kernels") or {}).items():      # a second kernel profiled on the same workload
+            if kernel and str(name).startswith(kernel):
+                rec = other
         total = float(rec["fetch_bytes"]) + float(rec["write_bytes"])
-    except (OSError, ValueError, KeyError, TypeError):
+    except (OSError, ValueError, KeyError, TypeError, AttributeError):
         return None, None
     source = dict(file=rel, kernel=rec.get("kernel"), kernel_sources_sha16=rec.get("kernel_sources_sha16"),
                   recorded_at_commit=rec.get("commit"))
