@@ -178,7 +178,7 @@ def other_config(torch, cs, config, stream, precision=None):
     abytes, flops = algorithmic_bytes(A.M, A.K, N, A.nnz), 2.0 * A.nnz * N
     ms, kernel_ms = timed_steps(torch, plan, dBs, dCs, steps, 5 if big else 50, 30.0, stream)
     kernels, dominant = plan_kernels(plan)
-    traffic, source = recorded_traffic(cfg["name"], dominant) if precision is None else (None, None)
+    traffic, source = recorded_traffic(cfg["name"], dominant)
     res = dict(workload=cfg["name"], M=A.M, K=A.K, N=N, nnz=A.nnz, kernel=dominant, kernels_per_step=kernels,
                precision=precision or "fp32", buffer_sets=R, steps=steps, us_per_step=ms * 1e3, kernel_us=kernel_ms * 1e3,
                value=flops / (ms * 1e-3) / 1e9, unit="GFLOP/s", algorithmic_bytes=abytes,
