@@ -1,6 +1,6 @@
 // run_cute -- single-GPU driver, the counterpart of the reference's main (run.cu:8-72).
 //
-//   run_cute <file.mtx | gen:CFG>  [--n 32,128,512] [--iters 20] [--keep-values] [--no-check] [--cache FILE]
+//   run_cute <file.mtx | gen:CFG>  [--n 32,128,512] [--iters 20] [--keep-values] [--no-check] [--cache FILE] [--extras]
 //
 // Reads (or generates) A, builds the HRPB once (timed, run.cu:17-20; with --cache the converted
 // matrix is written to FILE, and read from it instead when FILE already exists), fills B with seeded
@@ -8,6 +8,10 @@
 // plans, launches, times with HIP events (3 warm-ups, then `iters` launches inside one event pair) and --
 // the ERROR_CHECK branch of run.cu:57-64 -- compares with the plain CSR kernel.  One JSON
 // line per N on stdout: GFLOP/s = 2 nnz N / t, algorithmic GB/s and its share of 8 TB/s.
+// --extras also takes the two routes the reference's driver does not have, per N: the format built on the device from
+// the CSR arrays that live there (HRPB_DEVICE; its product, run with the partial tiles in a caller's buffer, must equal
+// the first one bit for bit) and the hybrid of inc/SPMM.cuh:2528-2933 (HybridSpMM: heavy tiles on the matrix cores,
+// the remainder on the row kernel; checked with the reference's metric).
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -46,7 +50,7 @@ int main(int argc, char **argv)
     std::vector<unsigned> widths = {32, 128, 512};
     int iters = 20;
     double ramp_ms = 30.0;     // launches before anything is timed: the GPU needs some milliseconds of work to reach its steady clocks
-    bool keep_values = false, check = true;
+    bool keep_values = false, check = true, extras = false;
     std::string cache_file;
     for (int i = 2; i < argc; ++i) {
         std::string a = argv[i];
@@ -57,6 +61,7 @@ int main(int argc, char **argv)
         else if (a == "--ramp-ms" && i + 1 < argc) ramp_ms = std::max(0.0, std::atof(argv[++i]));
         else if (a == "--keep-values") keep_values = true;
         else if (a == "--no-check") check = false;
+        else if (a == "--extras") extras = true;
         else if (a == "--cache" && i + 1 < argc) cache_file = argv[++i];
         else { std::fprintf(stderr, "unknown argument %s\n", a.c_str()); return 2; }
     }
@@ -154,16 +159,43 @@ int main(int argc, char **argv)
                 ref_metric = check_gemm_correctness_coo(c_ref.data(), c_host.data(), M, N);
                 back_err = cute_backward_error(hrpb.rowPtr, hrpb.cols, hrpb.vals, b.data(), c_ref.data(), c_host.data(), M, N);
             }
+            int device_built_equal = -1;
+            double hybrid_metric = -1.0;
+            unsigned hybrid_heavy = 0;
+            if (extras && check) {
+                const uint32_t *dRowPtr = nullptr, *dCols = nullptr;
+                const float *dVals = nullptr;
+                cute::check(cute_hrpb_dev_csr(hrpb.device, &dRowPtr, &dCols, &dVals), "cute_hrpb_dev_csr");
+                HRPB_DEVICE on_device(M, K, nnz, dRowPtr, dCols, dVals);
+                SPMM_TC spmm2(M, K, N, on_device);
+                DeviceBuffer dC3(size_t(M) * N), scratch(size_t(spmm2.scratch_bytes() / sizeof(float)) + 64);
+                spmm2.run(dB.p, dC3.p, nullptr, scratch.p, spmm2.scratch_bytes());
+                std::vector<float> c3(size_t(M) * N);
+                if (hipMemcpy(c3.data(), dC3.p, c3.size() * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
+                    throw cute::Error(CUTE_ERR_HIP, "hipMemcpy C (device-built)");
+                device_built_equal = std::memcmp(c3.data(), c_host.data(), c3.size() * sizeof(float)) == 0 ? 1 : 0;
+                SparseCoo<float> coo(static_cast<int>(M), static_cast<int>(K), static_cast<int>(nnz));
+                for (unsigned r = 0; r < M; ++r)
+                    for (unsigned e = hrpb.rowPtr[r]; e < hrpb.rowPtr[r + 1]; ++e) coo.Insert_Next(int(r), int(hrpb.cols[e]), hrpb.vals[e]);
+                CSR_Matrix<float> csr(coo);
+                HybridSpMM hybrid(&csr);
+                hybrid.run(dB.p, dC3.p, N);
+                if (hipMemcpy(c3.data(), dC3.p, c3.size() * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
+                    throw cute::Error(CUTE_ERR_HIP, "hipMemcpy C (hybrid)");
+                hybrid_metric = check_gemm_correctness_coo(c_ref.data(), c3.data(), M, N);
+                hybrid_heavy = hybrid.info.heavyTiles;
+            }
             const double flops = 2.0 * double(nnz) * N;
             const double bytes = double(nnz) * 8 + (double(M) + 1) * 4 + double(K) * N * 4 + double(M) * N * 4;
             std::printf("{\"matrix\": \"%s\", \"M\": %u, \"K\": %u, \"nnz\": %u, \"N\": %u, \"blocks\": %u, \"bricks\": %u, "
                         "\"brick_density\": %.4f, \"prep_ms\": %.3f, \"from_cache\": %s, \"chunks\": %u, \"atomic_chunks\": %u, \"sparse_panels\": %u, "
                         "\"kernel_us\": %.2f, \"gflops\": %.1f, \"algorithmic_GBps\": %.1f, \"hbm_roofline_frac\": %.4f, "
-                        "\"csr_kernel_us\": %.2f, \"max_rel_err\": %.3e, \"backward_err\": %.3e}\n",
+                        "\"csr_kernel_us\": %.2f, \"max_rel_err\": %.3e, \"backward_err\": %.3e, "
+                        "\"device_built_equal\": %d, \"hybrid_max_rel_err\": %.3e, \"hybrid_heavy_tiles\": %u}\n",
                         src.c_str(), M, K, nnz, N, hrpb.host().numBlocks, hrpb.num_bricks, hrpb.block_density, prep_ms, from_cache ? "true" : "false",
                         spmm.info.numChunks, spmm.info.numAtomicChunks, spmm.info.numRowPanelsSparse, t_ms * 1e3,
                         flops / (t_ms * 1e-3) / 1e9, bytes / (t_ms * 1e-3) / 1e9, bytes / (t_ms * 1e-3) / 8e12,
-                        csr_ms * 1e3, ref_metric, back_err);
+                        csr_ms * 1e3, ref_metric, back_err, device_built_equal, hybrid_metric, hybrid_heavy);
             std::fflush(stdout);
         }
         delete format;

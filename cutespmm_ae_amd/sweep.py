@@ -39,7 +39,7 @@ def find_matrices(root):
     return found
 
 
-def run_one(path, widths, iters, cache=None, check=True):
+def run_one(path, widths, iters, cache=None, check=True, extras=False):
     if not os.path.isfile(DRIVER):
         raise RuntimeError("run_cute is not built; run python -m cutespmm_ae_amd.build")
     cmd = [DRIVER, path, "--n", ",".join(str(n) for n in widths), "--iters", str(iters)]
@@ -47,6 +47,8 @@ def run_one(path, widths, iters, cache=None, check=True):
         cmd += ["--cache", cache]
     if not check:
         cmd.append("--no-check")
+    if extras:
+        cmd.append("--extras")      # also the device-built format and the hybrid call, per width
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("%s: %s" % (path, proc.stderr.strip() or "exit %d" % proc.returncode))

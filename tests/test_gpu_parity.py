@@ -622,6 +622,21 @@ def test_driver_and_sweep_tool(cs, torch_cuda, tmp_path):
     assert text.splitlines()[0] == "matrix, N(feature size), cuTeSpMM GFLOPS, CSR GFLOPS" and len(text.splitlines()) == 4
 
 
+def test_driver_extras_through_the_cpp_mirror(cs, torch_cuda):
+    """`run_cute --extras`: the C++ classes HRPB_DEVICE (format built on the device from CSR arrays that live there),
+    SPMM_TC::run with a caller's scratch buffer and HybridSpMM, on the golden matrix and on the R-MAT benchmark
+    matrix (cut panels: the scratch buffer is used).  The device-built format's product must equal the
+    host-built one's bit for bit; the hybrid is held to the reference's metric."""
+    import os
+    from cutespmm_ae_amd import sweep
+    from test_oracle_pins import GOLD
+    rows = sweep.run_one(os.path.join(GOLD, "G67.mtx"), [32, 100], 3, extras=True) + sweep.run_one("gen:4", [64], 3, extras=True)
+    assert [r["N"] for r in rows] == [32, 100, 64] and rows[2]["atomic_chunks"] > 0
+    for r in rows:
+        assert r["device_built_equal"] == 1, r
+        assert 0 <= r["hybrid_max_rel_err"] <= 1e-5 and r["max_rel_err"] <= 1e-5, r
+
+
 @pytest.mark.parametrize("block_size", [16, 32])
 def test_blocked_ell_spmm(cs, orc, torch_cuda, block_size):
     """Blocked-ELL device SpMM against the CSR oracle: random values (tolerance), integer values
