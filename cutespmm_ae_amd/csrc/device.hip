@@ -824,6 +824,25 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;
     }
+    // A handful of MFMA panels among row-kernel panels (the boundary panels of a stencil at N = 32: 64 of 16 384) would
+    // turn the launch into the fused kernel for their sake, which costs the row blocks more than those panels gain
+    // (9-point stencil of 512 x 512 points, N = 32: 29.0 us against 24.4 with every panel on the row kernel): when
+    // the MFMA panels hold less than 2 % of the entries and none of them has a row too long for a lane group,
+    // they go to the row kernel as well.
+    if (t.path == CUTE_PATH_AUTO && n_brick && n_rows) {
+        uint64_t nnz_mfma = 0;
+        bool movable = true;
+        for (uint32_t q = 0; q < d->P; ++q)
+            if (!to_rows[q]) {
+                nnz_mfma += d->panelNnz[q];
+                movable = movable && d->panelMaxRow[q] <= max_row_for_rows;
+            }
+        if (movable && nnz_mfma * 50u < uint64_t(d->nnz)) {
+            std::fill(to_rows.begin(), to_rows.end(), uint8_t(1));
+            n_rows += n_brick;
+            n_brick = 0;
+        }
+    }
 
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;

@@ -426,6 +426,34 @@ def test_default_kernel_choice(cs, orc, torch_cuda):
         assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR
 
 
+def test_a_handful_of_mfma_panels_goes_to_the_row_kernel(cs, orc, torch_cuda):
+    """9-point stencil at N = 32: only the panels on the grid's boundary (fewer columns, more reuse) would pass the bar
+    for the matrix cores -- 16 of 1 024 -- and the fused launch they would cause costs the other panels more than they
+    gain, so the whole matrix goes to the row kernel.  A panel with a row too long for a lane group keeps its MFMA kernel
+    (and the plan its fused launch).  Same product either way."""
+    A = cs.gen_matrix(2, 0xC07E5B02, 128)
+    h = cs.HRPB(A.M, A.K, A.rowPtr, A.cols, A.vals)
+    B = np.random.default_rng(8).standard_normal((A.K, 32)).astype(np.float32)
+    ref = orc.spmm_csr(A.rowPtr, A.cols, A.vals, B)
+    out, plan = _run(cs, torch_cuda, h, B)
+    assert plan.kernel_name == "csr_rows_batched" and plan.info["numBrickPanels"] == 0 and plan.info["numRowPanelsSparse"] == A.M // 16
+    assert cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, out) <= BERR
+    forced, fplan = _run(cs, torch_cuda, h, B, path=cs.PATH_BRICK)
+    assert fplan.info["numBrickPanels"] == A.M // 16 and cs.backward_error(A.rowPtr, A.cols, A.vals, B, ref, forced) <= BERR
+    # the same matrix with one row of 64 entries: its panel cannot go to the row kernel, so the plan stays mixed
+    rp, cl, vl = np.asarray(A.rowPtr).copy(), np.asarray(A.cols), np.asarray(A.vals)
+    r, long_row = 4000, 64
+    cols2 = np.concatenate([cl[:rp[r]], np.arange(long_row, dtype=np.uint32) * 3, cl[rp[r + 1]:]])
+    vals2 = np.concatenate([vl[:rp[r]], np.ones(long_row, np.float32), vl[rp[r + 1]:]])
+    rp2 = rp.copy()
+    rp2[r + 1:] += np.uint32(long_row - (rp[r + 1] - rp[r]))
+    h2 = cs.HRPB(A.M, A.K, rp2, cols2, vals2)
+    ref2 = orc.spmm_csr(rp2, cols2, vals2, B)
+    out2, plan2 = _run(cs, torch_cuda, h2, B)
+    assert plan2.info["numBrickPanels"] >= 1 and plan2.info["numRowPanelsSparse"] >= A.M // 16 - 20, plan2.info
+    assert cs.backward_error(rp2, cols2, vals2, B, ref2, out2) <= BERR
+
+
 def test_wide_products_of_short_rows_go_to_the_quad_kernel(cs, orc, torch_cuda):
     """50 000 rows of 7 entries at random columns: no reuse for the matrix cores to harvest, and at N = 128 the row
     kernel keeps them; at N = 512 the launch is several times the device and the quad kernel's deeper pipeline wins
@@ -620,6 +648,24 @@ def test_driver_and_sweep_tool(cs, torch_cuda, tmp_path):
             assert r["gflops"] > 0 and r["max_rel_err"] <= 1e-5 and r["backward_err"] <= BERR
     text = sweep.table([("G67", r) for r in first])
     assert text.splitlines()[0] == "matrix, N(feature size), cuTeSpMM GFLOPS, CSR GFLOPS" and len(text.splitlines()) == 4
+
+
+def test_sweep_kernel_durations_from_rocprofv3(cs, torch_cuda):
+    """The sweep tool's --rocprof column: one (matrix, N) under rocprofv3 --kernel-trace --stats, the plan's kernels
+    of one step added up and the CSR comparison kernel, against the driver's own event times."""
+    import os
+    import shutil
+    from cutespmm_ae_amd import sweep
+    from test_oracle_pins import GOLD
+    if not (shutil.which("rocprofv3") or os.path.exists("/opt/rocm/bin/rocprofv3")):
+        pytest.skip("rocprofv3 is not installed")
+    mtx = os.path.join(GOLD, "G67.mtx")
+    events = sweep.run_one(mtx, [128], 20)[0]
+    plan_us, csr_us = sweep.kernel_durations(mtx, 128, 20)
+    # kernel durations leave out what the event bracket adds per launch, so they are the smaller figures
+    assert 0 < plan_us <= 1.5 * events["kernel_us"] and 0 < csr_us <= 1.5 * events["csr_kernel_us"]
+    text = sweep.table([("G67", dict(events, kernel_us_rocprof=plan_us, csr_kernel_us_rocprof=csr_us))], rocprof=True)
+    assert text.splitlines()[1].startswith("G67, 128, ")
 
 
 def test_driver_extras_through_the_cpp_mirror(cs, torch_cuda):
