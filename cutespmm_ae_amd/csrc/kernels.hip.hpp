@@ -109,11 +109,13 @@ __device__ __forceinline__ void load_operands(BlockOperands<VEC, NG> &o, const B
         const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), 0u));
         o.a[j] = vals[hd.voff[j] + below];       // masked when consumed, so nothing waits here
         o.bitmap[j] = bm;
-        const float *brow = B + size_t(cols[j]) * N + col0;
+        const float *brow = B + size_t(cols[j]) * N;
 #pragma unroll
         for (int ng = 0; ng < NG; ++ng) {
-            if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) o.b[j][ng] = *reinterpret_cast<const V *>(brow + ng * 16 * VEC);
-            else o.b[j][ng] = V(0.0f);
+            // lanes beyond column N re-read the row's last VEC columns (N is a multiple of VEC) and store nothing:
+            // a branch around the load would split the pipeline's basic blocks
+            const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
+            o.b[j][ng] = *reinterpret_cast<const V *>(brow + ((FULL || c < N) ? c : N - VEC));
         }
     }
 }
@@ -296,23 +298,40 @@ __device__ __forceinline__ LeanHeader load_lean_header(const uint32_t *__restric
     return r;
 }
 
+// col_offs[ng]: byte offset inside a B row of the lane's VEC columns in column group ng.  When N is not a multiple of
+// the slab width, the lanes of the last slab that stand beyond column N point at the row's last VEC columns instead
+// (N is a multiple of VEC): they load valid memory, compute values nobody stores, and the loop keeps the one basic
+// block per iteration that its pipeline needs -- a branch around those loads cost 29 % (N = 192 against N = 256).
+template <int VEC, int NG, bool FULL>
+__device__ __forceinline__ void brick_column_offsets(uint32_t (&col_offs)[NG], uint32_t col0, uint32_t N)
+{
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng) {
+        const uint32_t c = col0 + uint32_t(ng) * 16u * VEC;
+        col_offs[ng] = ((FULL || c < N) ? c : N - VEC) * 4u;
+    }
+}
+
 template <int VEC, int NG, bool FULL>
 __device__ __forceinline__ void load_brick_lean(typename Vec<VEC>::type (&b_out)[NG], float &a_out, int j,
                                                 const LeanHeader &hd, const float *__restrict__ vals,
                                                 uint32_t zero_index, const float *__restrict__ B, uint32_t row_pitch,
-                                                uint32_t col_off, uint32_t col0, uint32_t N)
+                                                const uint32_t (&col_offs)[NG])
 {
     typedef typename Vec<VEC>::type V;
     const uint64_t bm = hd.bitmap[j];
     const uint32_t rank = __builtin_amdgcn_mbcnt_hi(uint32_t(bm >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(bm), hd.voff[j]));
     const uint32_t aoff = (__builtin_amdgcn_inverse_ballot_w64(bm) ? rank : zero_index) * 4u;
     a_out = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(vals) + aoff);
-    const uint32_t boff = __umul24(hd.cols[j], row_pitch) + col_off;
-    const char *brow = reinterpret_cast<const char *>(B) + boff;
+    const uint32_t row = __umul24(hd.cols[j], row_pitch);
+    if constexpr (FULL) {       // one address, the column groups at constant offsets from it
+        const char *brow = reinterpret_cast<const char *>(B) + (row + col_offs[0]);
 #pragma unroll
-    for (int ng = 0; ng < NG; ++ng) {
-        if (FULL || col0 + uint32_t(ng) * 16u * VEC < N) b_out[ng] = *reinterpret_cast<const V *>(brow + ng * 64 * VEC);
-        else b_out[ng] = V(0.0f);
+        for (int ng = 0; ng < NG; ++ng) b_out[ng] = *reinterpret_cast<const V *>(brow + ng * 64 * VEC);
+    } else {
+#pragma unroll
+        for (int ng = 0; ng < NG; ++ng)
+            b_out[ng] = *reinterpret_cast<const V *>(reinterpret_cast<const char *>(B) + (row + col_offs[ng]));
     }
 }
 
@@ -357,7 +376,9 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
     const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, block_x, block_y);
     if (!it.valid) return;
     const uint32_t end = it.end;
-    const uint32_t row_pitch = N * 4u, col_off = it.col0 * 4u;
+    const uint32_t row_pitch = N * 4u;
+    uint32_t col_offs[NG];
+    brick_column_offsets<VEC, NG, FULL>(col_offs, it.col0, N);
 
     f32x4 acc[NG][VEC];
 #pragma unroll
@@ -382,7 +403,7 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
             asm volatile("" ::"v"(h1.cols[0]), "v"(h1.cols[1]), "v"(h1.cols[2]), "v"(h1.cols[3]));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_offs);
                 bitmap[j] = h0.bitmap[j];
             }
         }
@@ -400,7 +421,7 @@ __device__ __forceinline__ void brick_rolling_body(uint32_t block_x, uint32_t bl
                     for (int v = 0; v < VEC; ++v)
                         acc[ng][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], vec_get<VEC>(b[j][ng], v), acc[ng][v], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+                load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_offs);
                 bitmap[j] = h1.bitmap[j];
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -499,7 +520,9 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 6 : 4)) void 
     const BrickItem it = brick_item<VEC, NG>(chunks, num_chunks, groups_per_xcd, lane, blockIdx.x, blockIdx.y);
     if (!it.valid) return;
     const uint32_t end = it.end;
-    const uint32_t row_pitch = N * 4u, col_off = it.col0 * 4u;
+    const uint32_t row_pitch = N * 4u;
+    uint32_t col_offs[NG];
+    brick_column_offsets<VEC, NG, FULL>(col_offs, it.col0, N);
 
     f32x4 acc[NG][VEC];
 #pragma unroll
@@ -517,7 +540,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 6 : 4)) void 
             h1 = load_lean_header(hdr, min(blk + 1, end - 1), lane);
             asm volatile("" ::"v"(h1.cols[0]), "v"(h1.cols[1]), "v"(h1.cols[2]), "v"(h1.cols[3]));   // as in the fp32 kernel
 #pragma unroll
-            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h0, vals, zero_index, B, row_pitch, col_offs);
         }
         Bf16Operands<NG> o;
         // per block: split what has arrived, ask for the next block into the same registers, multiply
@@ -527,7 +550,7 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 6 : 4)) void 
             split_block<NG>(o, a, b);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_off, it.col0, N);
+            for (int j = 0; j < 4; ++j) load_brick_lean<VEC, NG, FULL>(b[j], a[j], j, h1, vals, zero_index, B, row_pitch, col_offs);
             __builtin_amdgcn_sched_barrier(0);
             mfma_block_bf16x3<NG>(o, acc);
             __builtin_amdgcn_sched_barrier(0);
