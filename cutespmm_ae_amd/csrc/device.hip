@@ -829,6 +829,9 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     // (9-point stencil of 512 x 512 points, N = 32: 29.0 us against 24.4 with every panel on the row kernel): when
     // the MFMA panels hold less than 2 % of the entries and none of them has a row too long for a lane group,
     // they go to the row kernel as well.
+    // The same the other way round: a few row-kernel panels among MFMA panels cost a second launch or the fused
+    // kernel (FEM benchmark matrix, 53 of 3 000 panels: N = 8 21.2 us against 11.0 with every panel on the brick
+    // kernel, N = 16 12.3 against 10.7, N = 24 16.7 against 14.0); below 2 % of the entries they join the others.
     if (t.path == CUTE_PATH_AUTO && n_brick && n_rows) {
         uint64_t nnz_mfma = 0;
         bool movable = true;
@@ -841,8 +844,17 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
             std::fill(to_rows.begin(), to_rows.end(), uint8_t(1));
             n_rows += n_brick;
             n_brick = 0;
+        } else if ((uint64_t(d->nnz) - nnz_mfma) * 50u < uint64_t(d->nnz)) {
+            for (uint32_t q = 0; q < d->P; ++q)
+                if (to_rows[q] && d->brp[q + 1] != d->brp[q]) to_rows[q] = 2;      // (empty panels stay: the row kernel zeroes their rows)
+            n_brick += n_rows;
+            n_rows = 0;
         }
     }
+    // (2 marks the panels that joined: the choice of the MFMA shape below is made on the panels that earned it)
+    std::vector<uint8_t> joined(d->P, 0);
+    for (uint32_t q = 0; q < d->P; ++q)
+        if (to_rows[q] == 2) { joined[q] = 1; to_rows[q] = 0; }
 
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
@@ -890,7 +902,7 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         const uint32_t lists = d->quadRows == 4 ? 4u : 1u;     // list units per panel
         uint64_t slots = 0, bricks = 0, blocks = 0;
         for (uint32_t q = 0; q < d->P; ++q)
-            if (!to_rows[q]) {
+            if (!to_rows[q] && !joined[q]) {
                 slots += uint64_t(d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u;
                 bricks += (d->panelCols[q] + 3u) / 4u;
                 blocks += d->brp[q + 1] - d->brp[q];

@@ -452,6 +452,18 @@ def test_a_handful_of_mfma_panels_goes_to_the_row_kernel(cs, orc, torch_cuda):
     out2, plan2 = _run(cs, torch_cuda, h2, B)
     assert plan2.info["numBrickPanels"] >= 1 and plan2.info["numRowPanelsSparse"] >= A.M // 16 - 20, plan2.info
     assert cs.backward_error(rp2, cols2, vals2, B, ref2, out2) <= BERR
+    # and the other way round: the FEM benchmark matrix at N = 16, where 53 of 3 000 panels (0.5 % of the entries) would go
+    # to the row kernel and cost a fused launch -- they join the brick kernel; a stricter bar that sends a good part
+    # of the panels to the row kernel keeps the plan mixed
+    F = cs.gen_config(3)
+    hf = cs.HRPB(F.M, F.K, F.rowPtr, F.cols, F.vals)
+    Bf = np.random.default_rng(9).standard_normal((F.K, 16)).astype(np.float32)
+    reff = orc.spmm_csr(F.rowPtr, F.cols, F.vals, Bf)
+    outf, planf = _run(cs, torch_cuda, hf, Bf)
+    assert planf.kernel_name == "hrpb_brick_f32_rolling" and planf.info["numRowPanelsSparse"] == 0, planf.info
+    assert cs.backward_error(F.rowPtr, F.cols, F.vals, Bf, reff, outf) <= BERR
+    shares = [cs.SPMM_TC(hf, 64, min_reuse=bar, max_row_nnz=200).info for bar in (1.6, 2.0, 2.4, 2.8, 3.2)]
+    assert any(i["numRowPanelsSparse"] > 100 and i["numBrickPanels"] > 100 for i in shares), [(i["numRowPanelsSparse"], i["numBrickPanels"]) for i in shares]
 
 
 def test_wide_products_of_short_rows_go_to_the_quad_kernel(cs, orc, torch_cuda):
