@@ -22,6 +22,8 @@ constexpr uint64_t kWideWindowBytes = 16ull << 20;   // ... whose window of B is
 constexpr float kWideReuse = 0.98f;          // ... the bar for products of 256 columns or more over large matrices (see cute_spmm_plan_create)
 constexpr uint32_t kMaxRowForRows = 48;
 constexpr uint32_t kMaxHubRows = 256;       // hub plans: B rows a work-group keeps in LDS (64 KiB of 256-byte pieces; two work-groups per CU)     // ... unless it holds a row longer than this: one lane group would serialise it
+constexpr uint32_t kUnevenRowFloor = 16;     // row kernel vs MFMA kernel: a panel whose longest row exceeds this and ...
+constexpr uint32_t kUnevenRowRatio = 2;      // ... this many mean rows of the panel goes to the MFMA kernel while rows share wavefronts
 constexpr float kHybridFill = 0.15f;         // cute_hybrid: a tile goes to the Blocked-ELL part from this fill on (threshold 0)
 constexpr uint64_t kSlotsPerBrick = 8;      // quad lists when the MFMA panels need fewer list slots per 16x4 brick, else brick tiles
 // B and C together larger than the Infinity Cache: whatever the caller does between launches, their rows come
@@ -803,6 +805,19 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     p->d = d;
     // classify panels
     std::vector<uint8_t> to_rows(d->P, 0);
+    // panels that go to the MFMA kernel for another reason than their reuse (below); the choice of the MFMA shape is
+    // made on the panels that earned it
+    std::vector<uint8_t> joined(d->P, 0);
+    // The row kernel gives a row N / VEC lanes; up to N = 128 several rows share a wavefront, which then takes as long
+    // as its longest row.  A panel whose longest row is more than twice its mean row (and longer than two batches of
+    // eight entries) keeps its wavefronts waiting for that one row, and the MFMA kernel, which walks the panel's
+    // columns whatever row they belong to, is ahead although the reuse is low: on the reference's matrices with
+    // long-tailed rows (jan99jac*, de2010, ri2010, Wordnet3, bayer04, ted_B: 99th percentile of the row lengths 3-6 times
+    // the mean) 25-35 % at N = 16 and 32, geomean over the 43 matrices against the best single kernel 1.18 -> 1.10
+    // (N = 16), 1.10 -> 1.04 (N = 32), 1.07 -> 1.03 (N = 128).  With one row per wavefront (N >= 256) the same move
+    // loses (HEP-th-new, N = 512: 60 -> 68 us), so it is not made there.
+    const uint32_t row_lane_width = (N % 4 == 0) ? 4u : (N % 2 == 0) ? 2u : 1u;      // floats per lane of the row kernel
+    const bool rows_share_a_wavefront = t.max_row_nnz == 0 && (N + row_lane_width - 1u) / row_lane_width < 64u;
     uint32_t n_brick = 0, n_rows = 0, n_empty = 0;
     for (uint32_t q = 0; q < d->P; ++q) {
         const uint32_t nblk = d->brp[q + 1] - d->brp[q];
@@ -820,6 +835,11 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
             const uint32_t fetches = std::max(d->panelCols[q], (d->qgp[(q + 1) * lists] - d->qgp[q * lists]) * 16u);
             const float bar = (wide_and_large && uint64_t(d->panelSpan[q]) * N * sizeof(float) > kWideWindowBytes) ? kWideReuse : reuse_bar;
             rows = float(d->panelNnz[q]) < bar * float(fetches) && d->panelMaxRow[q] <= max_row_for_rows;
+            if (rows && rows_share_a_wavefront && d->panelMaxRow[q] > kUnevenRowFloor &&
+                uint64_t(d->panelMaxRow[q]) * CUTE_TM > uint64_t(kUnevenRowRatio) * d->panelNnz[q]) {
+                rows = false;
+                joined[q] = 1;
+            }
         }
         to_rows[q] = rows;
         if (nblk) (rows ? n_rows : n_brick)++;
@@ -846,15 +866,11 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
             n_brick = 0;
         } else if ((uint64_t(d->nnz) - nnz_mfma) * 50u < uint64_t(d->nnz)) {
             for (uint32_t q = 0; q < d->P; ++q)
-                if (to_rows[q] && d->brp[q + 1] != d->brp[q]) to_rows[q] = 2;      // (empty panels stay: the row kernel zeroes their rows)
+                if (to_rows[q] && d->brp[q + 1] != d->brp[q]) { to_rows[q] = 0; joined[q] = 1; }   // (empty panels stay: the row kernel zeroes their rows)
             n_brick += n_rows;
             n_rows = 0;
         }
     }
-    // (2 marks the panels that joined: the choice of the MFMA shape below is made on the panels that earned it)
-    std::vector<uint8_t> joined(d->P, 0);
-    for (uint32_t q = 0; q < d->P; ++q)
-        if (to_rows[q] == 2) { joined[q] = 1; to_rows[q] = 0; }
 
     // brick kernel shape
     p->vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
@@ -1156,7 +1172,7 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     p->info.pipeline = uint32_t(p->pipeline);
     // one launch for a mixed plan: the quad kernel with any row shape of 4-float lanes, the rolling brick
     // kernel in the shapes the planner itself picks for N (forced column groups fall back to two launches)
-    const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4 && p->rows_logl >= 2;
+    const bool rows_fusable = !chunks.empty() && !row_list.empty() && p->rows_vec == 4;
     const bool brick_default_shape = ng_for_mixed || p->ng == ((p->vec == 4 && N >= 128) ? 2 : 1);
     p->info.partialTileKiB = uint32_t((p->partialBytes + 1023u) / 1024u);
     p->info.fusedLaunch = (rows_fusable && !p->bf16x3 && !p->numHub && (p->shape == 2 || (p->pipeline == 1 && brick_default_shape))) ? 1u : 0u;
@@ -1347,7 +1363,9 @@ bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, floa
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs);
     if (uint64_t(grid.x) * grid.y + uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd >= 0x7fffffffull) return false;
     const int v = p->vec, g = p->ng, l = p->rows_logl;
-    if (v == 1 && g == 1 && l == 2) launch_brick_rows_as<1, 1, 2>(p, dB, dC, partials, s, grid, per_xcd);
+    if (v == 1 && g == 1 && l == 0) launch_brick_rows_as<1, 1, 0>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 1 && g == 1 && l == 1) launch_brick_rows_as<1, 1, 1>(p, dB, dC, partials, s, grid, per_xcd);
+    else if (v == 1 && g == 1 && l == 2) launch_brick_rows_as<1, 1, 2>(p, dB, dC, partials, s, grid, per_xcd);
     else if (v == 2 && g == 1 && l == 3) launch_brick_rows_as<2, 1, 3>(p, dB, dC, partials, s, grid, per_xcd);
     else if (v == 4 && g == 1 && l == 4) launch_brick_rows_as<4, 1, 4>(p, dB, dC, partials, s, grid, per_xcd);
     else if (v == 4 && g == 1 && l == 5) launch_brick_rows_as<4, 1, 5>(p, dB, dC, partials, s, grid, per_xcd);
@@ -1395,6 +1413,8 @@ int run_with(const cute_spmm_plan *p, const float *dB, float *dC, void *stream, 
                        partials, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \
+        case 0: CUTE_FUSED_LAUNCH(F, S, 0); break;                              \
+        case 1: CUTE_FUSED_LAUNCH(F, S, 1); break;                              \
         case 2: CUTE_FUSED_LAUNCH(F, S, 2); break;                              \
         case 3: CUTE_FUSED_LAUNCH(F, S, 3); break;                              \
         case 4: CUTE_FUSED_LAUNCH(F, S, 4); break;                              \

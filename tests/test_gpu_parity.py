@@ -466,6 +466,28 @@ def test_a_handful_of_mfma_panels_goes_to_the_row_kernel(cs, orc, torch_cuda):
     assert any(i["numRowPanelsSparse"] > 100 and i["numBrickPanels"] > 100 for i in shares), [(i["numRowPanelsSparse"], i["numBrickPanels"]) for i in shares]
 
 
+def test_panels_with_one_long_row_leave_the_row_kernel_at_narrow_widths(cs, orc, torch_cuda):
+    """Rows of 3 entries with one row of 40 in every other panel, all at random columns (no reuse for the matrix cores):
+    up to N = 128 several rows share a wavefront of the row kernel, which would wait for the long one, so those panels go
+    to the MFMA kernel; at N = 256 (one row per wavefront) and for evenly long rows (all 40) they stay."""
+    rng = np.random.default_rng(12)
+    M, K = 4096, 16384
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 40 if r % 32 == 5 else 3)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for N, uneven_to_mfma in ((32, True), (128, True), (256, False)):
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        out, plan = _run(cs, torch_cuda, h, B)
+        if uneven_to_mfma:
+            assert plan.info["numBrickPanels"] == M // 32 and plan.info["numRowPanelsSparse"] == M // 32, (N, plan.info)
+        else:
+            assert plan.info["numBrickPanels"] == 0, (N, plan.info)
+        assert cs.backward_error(rp, cl, vl, B, orc.spmm_csr(rp, cl, vl, B), out) <= BERR
+        # the caller's own limit on row lengths switches the rule off
+        assert cs.SPMM_TC(h, N, max_row_nnz=48).info["numBrickPanels"] == 0
+    rp2, cl2, vl2 = random_csr(rng, 1024, K, row_nnz=40)
+    assert cs.SPMM_TC(cs.HRPB(1024, K, rp2, cl2, vl2), 32).info["numBrickPanels"] == 0
+
+
 def test_wide_products_of_short_rows_go_to_the_quad_kernel(cs, orc, torch_cuda):
     """50 000 rows of 7 entries at random columns: no reuse for the matrix cores to harvest, and at N = 128 the row
     kernel keeps them; at N = 512 the launch is several times the device and the quad kernel's deeper pipeline wins
@@ -862,7 +884,7 @@ def test_strip_layout_of_the_quad_kernel(cs, orc, torch_cuda):
 
 def test_mixed_plans_at_narrow_widths(cs, orc, torch_cuda):
     """Dense panels next to sparse ones, so the planner mixes the MFMA and the row kernel: one fused
-    launch from 16 columns on (also for 4 and 8 lanes per row), narrow brick tiles for N <= 32."""
+    launch whenever N is a multiple of 4 (from one lane per row on), narrow brick tiles for N <= 32."""
     rng = np.random.default_rng(33)
     M, K = 640, 2048
     dense_rows = set(range(64, 160)) | set(range(400, 432))
@@ -880,7 +902,7 @@ def test_mixed_plans_at_narrow_widths(cs, orc, torch_cuda):
             info = plan.info
             assert info["numChunks"] > 0 and info["numRowPanelsSparse"] > 0, (N, kw, info)
             assert cs.backward_error(rp, cl, vl, B, ref, out) <= BERR, (N, kw, info)
-            assert info["fusedLaunch"] == (1 if N % 4 == 0 and N >= 12 else 0), (N, info)   # from 4 lanes per row on
+            assert info["fusedLaunch"] == (1 if N % 4 == 0 else 0), (N, info)   # whenever the row kernel's lanes hold four floats
             if info["mfmaShape"] == 1:
                 vec = 4 if N % 4 == 0 else 2 if N % 2 == 0 else 1
                 while vec > 1 and 8 * vec >= N:         # the narrowest tile that still covers N
