@@ -347,6 +347,16 @@ __global__ __launch_bounds__(kThreads) void quad_heads(const uint4 *__restrict__
     heads[id] = v;
 }
 
+// The row kernel's list of a mixed plan: every listed row with its row pointers, {row, first entry, end, 0}.
+__global__ __launch_bounds__(kThreads) void pack_row_list(const uint32_t *__restrict__ rows, uint32_t numRows,
+                                                          const uint32_t *__restrict__ rowPtr, uint4 *__restrict__ out)
+{
+    const uint64_t i = global_id();
+    if (i >= numRows) return;
+    const uint32_t r = rows[i];
+    out[i] = make_uint4(r, rowPtr[r], rowPtr[r + 1u], 0u);
+}
+
 // Hub plans (hrpb_quad_hub_f32): how often every column occurs in the quad records, and a copy of the records in
 // which the columns that have a slot in the LDS table of hub rows (slot_of[col] != ~0u) name that slot instead.
 __global__ __launch_bounds__(kThreads) void count_record_columns(const uint32_t *__restrict__ recs, uint64_t numGroups,

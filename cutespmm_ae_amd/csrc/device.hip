@@ -209,7 +209,7 @@ struct cute_spmm_plan {
     float *dPartials = nullptr;         // pieces x unitRows rows of N floats; owned by the plan, so a plan runs on one stream at a time
     uint64_t partialBytes = 0;
     void *staticScratch = nullptr;      // device address of the library's static scratch array on the plan's device
-    uint32_t *dRowList = nullptr;
+    uint4 *dRowList = nullptr;          // rows of the sparse path with their row pointers: {row, first entry, end, 0}
     uint32_t numRows = 0;
     cute_dev::XcdRanges rowRanges{};   // row-kernel blocks of each XCD, balanced by nonzeros
     uint32_t rowBlocksPerXcd = 0;       // longest of those ranges
@@ -1147,7 +1147,19 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         p->partialBytes = bytes;
         if (hipMalloc(reinterpret_cast<void **>(&p->dPartials), bytes) != hipSuccess) rc = CUTE_ERR_NOMEM;
     }
-    if (rc == CUTE_OK) rc = upload(&p->dRowList, row_list.data(), row_list.size());
+    if (rc == CUTE_OK && !row_list.empty()) {
+        // the list goes up as row indices and is packed with the rows' pointers on the device, where those are
+        uint32_t *rows_only = nullptr;
+        rc = upload(&rows_only, row_list.data(), row_list.size());
+        if (rc == CUTE_OK && hipMalloc(reinterpret_cast<void **>(&p->dRowList), row_list.size() * sizeof(uint4)) != hipSuccess) rc = CUTE_ERR_NOMEM;
+        if (rc == CUTE_OK) {
+            hipLaunchKernelGGL(cute_build::pack_row_list, grid_of(row_list.size()), dim3(cute_build::kThreads), 0, nullptr, rows_only,
+                               uint32_t(row_list.size()), d->dRowPtr, p->dRowList);
+            rc = check_launch("row list");
+            if (rc == CUTE_OK && hipStreamSynchronize(nullptr) != hipSuccess) rc = CUTE_ERR_HIP;
+        }
+        (void)hipFree(rows_only);
+    }
     if (rc == CUTE_OK) {
         // cute_spmm_run_static's scratch: its address on this device is looked up here, at set-up, so that the
         // run call itself is nothing but kernel launches
@@ -1210,7 +1222,7 @@ void launch_brick(const cute_spmm_plan *p, const float *dB, float *dC, float *pa
 }
 
 template <int VEC, bool BATCHED>
-void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
+void launch_rows_vec(int logl, const uint4 *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
                      const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s,
                      const cute_dev::XcdRanges *ranges, uint32_t blocks_per_xcd)
 {
@@ -1225,7 +1237,7 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
             hipLaunchKernelGGL((cute_dev::csr_rows_batched<VEC, LL, 8>), grid, block, 0, s, row_list, num_rows,    \
                                slabs, rp, cl, vl, dB, dC, N, rg);                                                 \
         else                                                                                                      \
-            hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, row_list, num_rows, slabs, rp,    \
+            hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, static_cast<const uint32_t *>(nullptr), num_rows, slabs, rp, \
                                cl, vl, dB, dC, N);                                                                \
         break;
     switch (logl) {
@@ -1237,7 +1249,7 @@ void launch_rows_vec(int logl, const uint32_t *row_list, uint32_t num_rows, uint
 
 // batched: the library's sparse-panel kernel; otherwise the plain comparison kernel
 template <bool BATCHED>
-void launch_rows(int vec, int logl, const uint32_t *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
+void launch_rows(int vec, int logl, const uint4 *row_list, uint32_t num_rows, uint32_t slabs, const uint32_t *rp,
                  const uint32_t *cl, const float *vl, const float *dB, float *dC, uint32_t N, hipStream_t s,
                  const cute_dev::XcdRanges *ranges = nullptr, uint32_t blocks_per_xcd = 0)
 {

@@ -991,7 +991,7 @@ __global__ __launch_bounds__(256) void csr_rows(const uint32_t *__restrict__ row
 // row costs about one memory round trip per batch instead of one per nonzero.  Each C
 // element still accumulates its row in storage order.
 template <int VEC, int LOG_L, int BATCH>
-__device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint32_t *__restrict__ row_list, uint32_t num_rows,
+__device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint4 *__restrict__ row_list, uint32_t num_rows,
                                                   uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
                                                   const uint32_t *__restrict__ cols, const float *__restrict__ vals,
                                                   const float *__restrict__ B, float *__restrict__ C, uint32_t N)
@@ -1004,10 +1004,17 @@ __device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint3
     if (gid >= uint64_t(num_rows) * num_slabs) return;
     const uint32_t ridx = uint32_t(gid / num_slabs);
     const uint32_t slab = uint32_t(gid % num_slabs);
-    const uint32_t row = row_list ? row_list[ridx] : ridx;
+    // a listed row comes with its row pointers {row, first entry, end, -}: one fetch, where the row index in one array
+    // and the row pointers in another would be two, the second waiting for the first
+    uint32_t row, s, e;
+    if (row_list) {
+        const uint4 entry = row_list[ridx];
+        row = entry.x; s = entry.y; e = entry.z;
+    } else {
+        row = ridx; s = rowPtr[row]; e = rowPtr[row + 1];
+    }
     const uint32_t c0 = slab * L * VEC + t * VEC;
     const bool live = c0 < N;
-    const uint32_t s = rowPtr[row], e = rowPtr[row + 1];
     const float *bcol = B + c0;
     V acc = V(0.0f);
     for (uint32_t base = s; base < e; base += L) {
@@ -1035,7 +1042,7 @@ __device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint3
 }
 
 template <int VEC, int LOG_L, int BATCH>
-__global__ __launch_bounds__(256) void csr_rows_batched(const uint32_t *__restrict__ row_list, uint32_t num_rows,
+__global__ __launch_bounds__(256) void csr_rows_batched(const uint4 *__restrict__ row_list, uint32_t num_rows,
                                                         uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
                                                         const uint32_t *__restrict__ cols,
                                                         const float *__restrict__ vals, const float *__restrict__ B,
@@ -1057,7 +1064,7 @@ template <bool FULL, bool STRIPS, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
     uint32_t quad_blocks_x, uint32_t quad_blocks, const uint32_t *__restrict__ heads, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
-    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
     const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
@@ -1077,7 +1084,7 @@ template <int VEC, int NG, bool FULL, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_rows_f32(
     uint32_t brick_blocks_x, uint32_t brick_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ tile_vals, uint32_t zero_index,
-    const uint32_t *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
     const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
