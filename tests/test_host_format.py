@@ -6,6 +6,7 @@ import os
 import re
 
 import numpy as np
+import scipy.sparse
 import pytest
 
 from helpers import dense_from_csr, hrpb_check_invariants, random_csr
@@ -251,20 +252,29 @@ def test_generators_match_their_specification(cs):
     assert np.abs(A.vals).max() <= 1.0
     S = cs.gen_config(2)
     assert (S.M, S.nnz) == (65536, 766 * 766)
-    D = dense_from_csr(64 * 64, 64 * 64, *(lambda m: (m.rowPtr, m.cols, m.vals))(cs.gen_matrix(2, 5, 64)))
-    assert (np.abs(np.diag(D) - 8) <= 0.01).all()
-    off = D - np.diag(np.diag(D))
-    assert ((off == 0) | (np.abs(off + 1) <= 0.01)).all() and ((off != 0) == (off != 0).T).all()
+    def sparse(m):
+        return scipy.sparse.csr_matrix((m.vals.astype(np.float64), m.cols.astype(np.int64), m.rowPtr.astype(np.int64)), shape=(m.M, m.K))
+
+    def pattern_is_symmetric(a):
+        p = (a != 0).astype(np.int8)
+        return (p != p.T).nnz == 0
+
+    D = sparse(cs.gen_matrix(2, 5, 64))
+    assert D.shape == (64 * 64, 64 * 64) and (np.abs(D.diagonal() - 8) <= 0.01).all()
+    off = (D - scipy.sparse.diags(D.diagonal())).tocsr()
+    off.eliminate_zeros()
+    assert (np.abs(off.data + 1) <= 0.01).all() and pattern_is_symmetric(off)
     F = cs.gen_config(3, 0.05)
-    Df = dense_from_csr(F.M, F.K, F.rowPtr, F.cols, F.vals)
-    assert ((Df != 0) == (Df != 0).T).all()
-    assert (np.abs(np.diag(Df)) > np.abs(Df).sum(1) - np.abs(np.diag(Df))).all()
+    Df = sparse(F)
+    assert pattern_is_symmetric(Df)
+    assert (np.abs(Df.diagonal()) > np.asarray(abs(Df).sum(1)).ravel() - np.abs(Df.diagonal())).all()
     R = cs.gen_config(4, 1 / 64.0)
-    Dr = dense_from_csr(R.M, R.K, R.rowPtr, R.cols, R.vals)
-    deg = (Dr != 0).sum(1)
-    assert (np.diag(Dr) > 0).all() and ((Dr != 0) == (Dr != 0).T).all()
-    i, j = np.nonzero(Dr)
-    assert np.allclose(Dr[i, j], 1 / np.sqrt(deg[i] * deg[j]), rtol=1e-6)
+    Dr = sparse(R)
+    assert (Dr.data != 0).all()
+    deg = np.diff(Dr.indptr)
+    assert (Dr.diagonal() > 0).all() and pattern_is_symmetric(Dr)
+    i, j = Dr.nonzero()
+    assert np.allclose(np.asarray(Dr[i, j]).ravel(), 1 / np.sqrt(deg[i] * deg[j]), rtol=1e-6)
     Bd = cs.gen_config(5, 1 / 256.0)
     assert (np.diff(Bd.rowPtr.astype(np.int64)) == 32).all()
     rows = np.repeat(np.arange(Bd.M), 32)
