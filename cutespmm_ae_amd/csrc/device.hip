@@ -1030,8 +1030,8 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     // Row-kernel blocks per XCD: contiguous ranges of rows (neighbouring rows share B rows, which then stay
     // in one L2), cut where the running work -- nonzeros plus a fixed cost per row -- passes each eighth.
     {
-        const uint32_t items_per_block = 256u >> p->rows_logl;             // (row, slab) pairs of one 256-thread block
-        const uint64_t total_items = uint64_t(row_list.size()) * p->rows_slabs;
+        const uint32_t items_per_block = 256u >> p->rows_logl;             // rows of one 256-thread block (per slab)
+        const uint64_t total_items = uint64_t(row_list.size());
         const uint32_t total_blocks = uint32_t((total_items + items_per_block - 1) / items_per_block);
         uint64_t total_work = 0;
         for (uint32_t q = 0; q < d->P; ++q)
@@ -1042,7 +1042,7 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
         for (uint32_t q = 0; q < d->P && x < cute_dev::kNumXcd; ++q) {
             if (!to_rows[q]) continue;
             work += d->panelNnz[q] + 4u * CUTE_TM;
-            items += uint64_t(CUTE_TM) * p->rows_slabs;
+            items += uint64_t(CUTE_TM);
             while (x < cute_dev::kNumXcd && work * cute_dev::kNumXcd >= total_work * x)
                 p->rowRanges.first[x++] = uint32_t(std::min<uint64_t>(total_blocks, (items + items_per_block - 1) / items_per_block));
         }
@@ -1229,13 +1229,14 @@ void launch_rows_vec(int logl, const uint4 *row_list, uint32_t num_rows, uint32_
     const uint64_t lanes = (uint64_t(num_rows) * slabs) << logl;
     // the batched kernel deals its blocks to the XCDs in contiguous ranges (all as long as the longest)
     const uint32_t blocks = uint32_t((lanes + 255) / 256);
-    const dim3 grid(BATCHED ? blocks_per_xcd * cute_dev::kNumXcd : blocks), block(256);
+    // the batched kernel walks the slabs in the grid's y dimension; the plain one folds them into x
+    const dim3 grid(BATCHED ? blocks_per_xcd * cute_dev::kNumXcd : blocks, BATCHED ? slabs : 1u), block(256);
     const cute_dev::XcdRanges rg = ranges ? *ranges : cute_dev::XcdRanges{};
 #define CUTE_ROWS_CASE(LL)                                                                                        \
     case LL:                                                                                                      \
         if (BATCHED)                                                                                              \
             hipLaunchKernelGGL((cute_dev::csr_rows_batched<VEC, LL, 8>), grid, block, 0, s, row_list, num_rows,    \
-                               slabs, rp, cl, vl, dB, dC, N, rg);                                                 \
+                               rp, cl, vl, dB, dC, N, rg);                                                        \
         else                                                                                                      \
             hipLaunchKernelGGL((cute_dev::csr_rows<VEC, LL>), grid, block, 0, s, static_cast<const uint32_t *>(nullptr), num_rows, slabs, rp, \
                                cl, vl, dB, dC, N);                                                                \
@@ -1356,12 +1357,13 @@ void launch_brick_rows_as(const cute_spmm_plan *p, const float *dB, float *dC, f
                           uint32_t per_xcd)
 {
     const uint32_t N = p->info.N;
-    const uint64_t brick_blocks = uint64_t(grid.x) * grid.y, row_blocks = uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd;
+    const uint32_t rows_per_slab = p->rowBlocksPerXcd * cute_dev::kNumXcd;
+    const uint64_t brick_blocks = uint64_t(grid.x) * grid.y, row_blocks = uint64_t(rows_per_slab) * p->rows_slabs;
     const dim3 flat(uint32_t(brick_blocks + row_blocks)), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
 #define CUTE_BRICK_ROWS(F)                                                                                                \
     hipLaunchKernelGGL((cute_dev::hrpb_brick_rows_f32<VEC, NG, F, LOG_L>), flat, block, 0, s, grid.x, uint32_t(brick_blocks),  \
                        p->dChunks, p->info.numChunks, per_xcd, p->d->dHdr, p->d->dVals, uint32_t(p->d->numVals), p->dRowList, \
-                       p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals,                    \
+                       p->numRows, rows_per_slab, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals,                    \
                        dB, dC, partials, N)
     if (N % (16u * VEC * NG) == 0) CUTE_BRICK_ROWS(true);
     else CUTE_BRICK_ROWS(false);
@@ -1373,7 +1375,7 @@ bool launch_brick_rows(const cute_spmm_plan *p, const float *dB, float *dC, floa
     const uint32_t groups = (p->info.numChunks + cute_dev::kWavesPerGroup - 1) / cute_dev::kWavesPerGroup;
     const uint32_t per_xcd = (groups + cute_dev::kNumXcd - 1) / cute_dev::kNumXcd;
     const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs);
-    if (uint64_t(grid.x) * grid.y + uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd >= 0x7fffffffull) return false;
+    if (uint64_t(grid.x) * grid.y + uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd * p->rows_slabs >= 0x7fffffffull) return false;
     const int v = p->vec, g = p->ng, l = p->rows_logl;
     if (v == 1 && g == 1 && l == 0) launch_brick_rows_as<1, 1, 0>(p, dB, dC, partials, s, grid, per_xcd);
     else if (v == 1 && g == 1 && l == 1) launch_brick_rows_as<1, 1, 1>(p, dB, dC, partials, s, grid, per_xcd);
@@ -1415,13 +1417,14 @@ int run_with(const cute_spmm_plan *p, const float *dB, float *dC, void *stream, 
         const dim3 grid(per_xcd * cute_dev::kNumXcd, p->info.numSlabs), block(cute_dev::kWaveSize * cute_dev::kWavesPerGroup);
         const bool full = N % 64u == 0, strips = p->d->quadRows == 4;
         // mixed plan: quad chunks and sparse rows in one launch (instantiated for 4-float lanes and 4..64 lanes per row)
-        const uint64_t row_blocks = uint64_t(p->rowBlocksPerXcd) * cute_dev::kNumXcd, quad_blocks = uint64_t(grid.x) * grid.y;
+        const uint32_t rows_per_slab = p->rowBlocksPerXcd * cute_dev::kNumXcd;
+        const uint64_t row_blocks = uint64_t(rows_per_slab) * p->rows_slabs, quad_blocks = uint64_t(grid.x) * grid.y;
         if (p->info.fusedLaunch && quad_blocks + row_blocks < 0x7fffffffull) {
 #define CUTE_FUSED_LAUNCH(F, S, LL)                                                                                       \
     hipLaunchKernelGGL((cute_dev::hrpb_quad_rows_f32<F, S, LL>), dim3(uint32_t(quad_blocks + row_blocks)), block, 0, s,     \
                        grid.x, uint32_t(quad_blocks), p->dHeads, p->info.numChunks, per_xcd, p->d->dQRecs, p->d->dQVals,   \
                        uint32_t(p->d->numQuadVals),                                                                  \
-                       p->dRowList, p->numRows, p->rows_slabs, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC,    \
+                       p->dRowList, p->numRows, rows_per_slab, p->rowRanges, p->d->dRowPtr, p->d->dCols, p->d->dCsrVals, dB, dC,    \
                        partials, N)
 #define CUTE_FUSED_LL(F, S)                                                     \
     switch (p->rows_logl) {                                                     \

@@ -991,8 +991,8 @@ __global__ __launch_bounds__(256) void csr_rows(const uint32_t *__restrict__ row
 // row costs about one memory round trip per batch instead of one per nonzero.  Each C
 // element still accumulates its row in storage order.
 template <int VEC, int LOG_L, int BATCH>
-__device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint4 *__restrict__ row_list, uint32_t num_rows,
-                                                  uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+__device__ __forceinline__ void rows_batched_body(uint32_t block_id, uint32_t slab, const uint4 *__restrict__ row_list,
+                                                  uint32_t num_rows, const uint32_t *__restrict__ rowPtr,
                                                   const uint32_t *__restrict__ cols, const float *__restrict__ vals,
                                                   const float *__restrict__ B, float *__restrict__ C, uint32_t N)
 {
@@ -1001,9 +1001,8 @@ __device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint4
     constexpr uint32_t STEP = BATCH < int(L) ? uint32_t(BATCH) : L;
     const uint32_t t = threadIdx.x & (L - 1);
     const uint64_t gid = (uint64_t(block_id) * blockDim.x + threadIdx.x) >> LOG_L;
-    if (gid >= uint64_t(num_rows) * num_slabs) return;
-    const uint32_t ridx = uint32_t(gid / num_slabs);
-    const uint32_t slab = uint32_t(gid % num_slabs);
+    if (gid >= num_rows) return;
+    const uint32_t ridx = uint32_t(gid);
     // a listed row comes with its row pointers {row, first entry, end, -}: one fetch, where the row index in one array
     // and the row pointers in another would be two, the second waiting for the first
     uint32_t row, s, e;
@@ -1043,16 +1042,18 @@ __device__ __forceinline__ void rows_batched_body(uint32_t block_id, const uint4
 
 template <int VEC, int LOG_L, int BATCH>
 __global__ __launch_bounds__(256) void csr_rows_batched(const uint4 *__restrict__ row_list, uint32_t num_rows,
-                                                        uint32_t num_slabs, const uint32_t *__restrict__ rowPtr,
+                                                        const uint32_t *__restrict__ rowPtr,
                                                         const uint32_t *__restrict__ cols,
                                                         const float *__restrict__ vals, const float *__restrict__ B,
                                                         float *__restrict__ C, uint32_t N, XcdRanges ranges)
 {
     // each XCD walks one contiguous range of rows (ranges of equal work), so the B rows that neighbouring
-    // rows share stay in that XCD's L2
+    // rows share stay in that XCD's L2.  A product wider than one lane group's slab (2^LOG_L * VEC columns) is
+    // walked slab by slab, each over all rows (y is the slower index of the order in which work-groups start):
+    // what the resident rows read of B at one time is then one slab wide, whatever N is.
     uint32_t block_id;
     if (!xcd_range_id(ranges, blockIdx.x, block_id)) return;
-    rows_batched_body<VEC, LOG_L, BATCH>(block_id, row_list, num_rows, num_slabs, rowPtr, cols, vals, B, C, N);
+    rows_batched_body<VEC, LOG_L, BATCH>(block_id, blockIdx.y, row_list, num_rows, rowPtr, cols, vals, B, C, N);
 }
 
 // One launch for a plan that uses both the quad kernel and the row kernel: they write disjoint
@@ -1064,7 +1065,7 @@ template <bool FULL, bool STRIPS, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f32(
     uint32_t quad_blocks_x, uint32_t quad_blocks, const uint32_t *__restrict__ heads, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ qrecs, const float *__restrict__ qvals, uint32_t zero_index,
-    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_blocks_per_slab, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
     const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
@@ -1073,9 +1074,10 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, 8) void hrpb_quad_rows_f
         quad_body<FULL, STRIPS>(blockIdx.x % quad_blocks_x, blockIdx.x / quad_blocks_x, heads, num_chunks, groups_per_xcd,
                                 qrecs, qvals, zero_index, B, C, partials, N);
     } else {   // quad_blocks is a multiple of the XCD count, so the XCD of a row block is (its index) % 8 as well
+        const uint32_t rb = blockIdx.x - quad_blocks, slab = rb / row_blocks_per_slab;      // slab by slab, as in csr_rows_batched
         uint32_t block_id;
-        if (!xcd_range_id(row_ranges, blockIdx.x - quad_blocks, block_id)) return;
-        rows_batched_body<4, LOG_L, 8>(block_id, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
+        if (!xcd_range_id(row_ranges, rb - slab * row_blocks_per_slab, block_id)) return;
+        rows_batched_body<4, LOG_L, 8>(block_id, slab, row_list, num_rows, rowPtr, cols, vals, B, C, N);
     }
 }
 
@@ -1084,7 +1086,7 @@ template <int VEC, int NG, bool FULL, int LOG_L>
 __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void hrpb_brick_rows_f32(
     uint32_t brick_blocks_x, uint32_t brick_blocks, const uint4 *__restrict__ chunks, uint32_t num_chunks,
     uint32_t groups_per_xcd, const uint32_t *__restrict__ hdr, const float *__restrict__ tile_vals, uint32_t zero_index,
-    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_slabs, XcdRanges row_ranges,
+    const uint4 *__restrict__ row_list, uint32_t num_rows, uint32_t row_blocks_per_slab, XcdRanges row_ranges,
     const uint32_t *__restrict__ rowPtr, const uint32_t *__restrict__ cols, const float *__restrict__ vals,
     const float *__restrict__ B, float *__restrict__ C, float *__restrict__ partials, uint32_t N)
 {
@@ -1092,9 +1094,10 @@ __global__ __launch_bounds__(kWaveSize *kWavesPerGroup, (NG == 1 ? 8 : 4)) void 
         brick_rolling_body<VEC, NG, FULL>(blockIdx.x % brick_blocks_x, blockIdx.x / brick_blocks_x, chunks, num_chunks,
                                           groups_per_xcd, hdr, tile_vals, zero_index, B, C, partials, N);
     } else {
+        const uint32_t rb = blockIdx.x - brick_blocks, slab = rb / row_blocks_per_slab;
         uint32_t block_id;
-        if (!xcd_range_id(row_ranges, blockIdx.x - brick_blocks, block_id)) return;
-        rows_batched_body<4, LOG_L, 8>(block_id, row_list, num_rows, row_slabs, rowPtr, cols, vals, B, C, N);
+        if (!xcd_range_id(row_ranges, rb - slab * row_blocks_per_slab, block_id)) return;
+        rows_batched_body<4, LOG_L, 8>(block_id, slab, row_list, num_rows, rowPtr, cols, vals, B, C, N);
     }
 }
 
