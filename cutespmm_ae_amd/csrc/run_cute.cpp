@@ -5,7 +5,7 @@
 // Reads (or generates) A, builds the HRPB once (timed, run.cu:17-20; with --cache the converted
 // matrix is written to FILE, and read from it instead when FILE already exists), fills B with seeded
 // U(0,1) values (run.cu:24-27 uses rand()), then for every N (run.cu:16: 32, 128, 512)
-// plans, launches, times with HIP events (3 warm-ups, then `iters` launches inside one event pair) and --
+// plans, launches, times with HIP events (3 warm-ups, then `iters` launches inside one event pair, the median of three such pairs) and --
 // the ERROR_CHECK branch of run.cu:57-64 -- compares with the plain CSR kernel.  One JSON
 // line per N on stdout: GFLOP/s = 2 nnz N / t, algorithmic GB/s and its share of 8 TB/s.
 // --extras also takes the two routes the reference's driver does not have, per N: the format built on the device from
@@ -130,15 +130,22 @@ int main(int argc, char **argv)
                 for (int w = 0; w < 3; ++w) launch();
                 hipEvent_t e0, e1;
                 if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) throw cute::Error(CUTE_ERR_HIP, "hipEventCreate");
-                (void)hipEventRecord(e0, nullptr);
-                for (int it = 0; it < iters; ++it) launch();
-                (void)hipEventRecord(e1, nullptr);
-                float total_ms = 0.0f;
-                if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&total_ms, e0, e1) != hipSuccess)
-                    throw cute::Error(CUTE_ERR_HIP, "timing");
+                // three such brackets, the median reported: launches of a few microseconds scatter by 10-20 % from
+                // one bracket to the next
+                double bracket_ms[3];
+                for (double &ms : bracket_ms) {
+                    (void)hipEventRecord(e0, nullptr);
+                    for (int it = 0; it < iters; ++it) launch();
+                    (void)hipEventRecord(e1, nullptr);
+                    float total_ms = 0.0f;
+                    if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&total_ms, e0, e1) != hipSuccess)
+                        throw cute::Error(CUTE_ERR_HIP, "timing");
+                    ms = double(total_ms) / iters;
+                }
                 (void)hipEventDestroy(e0);
                 (void)hipEventDestroy(e1);
-                return double(total_ms) / iters;
+                std::sort(bracket_ms, bracket_ms + 3);
+                return bracket_ms[1];
             };
             const double t_ms = time_launches([&] { spmm.run(dB.p, dC.p); });
             double ref_metric = -1.0, back_err = -1.0, csr_ms = -1.0;
