@@ -205,6 +205,7 @@ struct cute_spmm_plan {
     // panels (or 4-row strips) cut into several chunks: each chunk stores a partial tile, reduce_partials adds them
     uint4 *dFixups = nullptr;           // {panel or strip, first piece, pieces, -}
     uint32_t numFixups = 0;
+    uint32_t reduceBlocksY = 1;         // blocks of reduce_partials along a tile: enough for the tile with the most pieces
     uint32_t unitRows = CUTE_TM;        // rows of one panel / strip / piece
     float *dPartials = nullptr;         // pieces x unitRows rows of N floats; owned by the plan, so a plan runs on one stream at a time
     uint64_t partialBytes = 0;
@@ -1139,8 +1140,18 @@ int cute_spmm_plan_create(cute_hrpb_dev *d, uint32_t N, const cute_tunables *tn,
     }
     if (rc == CUTE_OK) rc = upload(&p->dFixups, fixups.data(), fixups.size());
     p->unitRows = CUTE_TM / upp;
-    // reduce_partials walks a tile along grid.y
+    // reduce_partials walks a tile along grid.y, a block of sixteen wavefronts taking 16 / G segments of 64 elements, G = 1..16
+    // wavefronts to a segment by the number of pieces (see the kernel): the launch gets the blocks its tile with the most
+    // pieces needs (the others leave theirs early), not one per segment -- with thousands of cut panels of two or three
+    // pieces each the blocks that only start and exit otherwise cost more than the sums
     if (rc == CUTE_OK && n_pieces && (uint64_t(CUTE_TM / upp) * N + 63u) / 64u > 65535u) rc = CUTE_ERR_SHAPE;
+    {
+        uint32_t most = 1;
+        for (const uint4 &fx : fixups) most = std::max(most, fx.z);
+        const uint32_t G = most <= 4 ? 1u : most <= 8 ? 2u : most <= 16 ? 4u : most <= 32 ? 8u : 16u;    // as in reduce_partials
+        const uint32_t segments = (CUTE_TM / upp * N + 63u) / 64u, per_block = uint32_t(cute_dev::kReduceWaves) / G;
+        p->reduceBlocksY = std::max(1u, (segments + per_block - 1u) / per_block);
+    }
     if (rc == CUTE_OK && n_pieces) {
         // (the fast kernels address the partial tiles like C, with 32-bit byte offsets: checked where the chunks were made)
         const uint64_t bytes = uint64_t(n_pieces) * p->unitRows * N * sizeof(float);
@@ -1468,7 +1479,7 @@ int run_with(const cute_spmm_plan *p, const float *dB, float *dC, void *stream, 
     // panels that were cut: add their partial tiles up, in chunk order (no atomics, so a product is
     // the same bit for bit every time it is computed)
     if (p->numFixups)
-        hipLaunchKernelGGL(cute_dev::reduce_partials, dim3(p->numFixups, (p->unitRows * N + 63u) / 64u),
+        hipLaunchKernelGGL(cute_dev::reduce_partials, dim3(p->numFixups, p->reduceBlocksY),
                            dim3(cute_dev::kWaveSize * cute_dev::kReduceWaves), 0, s, p->dFixups, p->numFixups, p->unitRows,
                            partials, dC, N);
     return check_launch("spmm launch");
