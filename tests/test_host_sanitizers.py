@@ -16,7 +16,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "cutespmm_ae_amd", "csrc")
 HOST_UNITS = ["host_format.cpp", "host_formats2.cpp", "host_quad.cpp", "host_cache.cpp", "gen.cpp"]
-COMMON = ["-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer", "-pthread", "-I", os.path.join(ROOT, "include")]
+COMMON = ["-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer", "-pthread", "-ffp-contract=off", "-Wno-unknown-pragmas", "-I", os.path.join(ROOT, "include")]
 FLAVOURS = {
     # the address sanitizer's runtime is linked statically: a dynamic one insists on being the first library loaded
     "address+undefined": (["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"], ["-static-libasan"]),
