@@ -910,6 +910,39 @@ def test_mixed_plans_at_narrow_widths(cs, orc, torch_cuda):
                 assert info["slabWidth"] == 16 * vec * (2 if vec == 4 and N >= 128 else 1), (N, info)
 
 
+def test_mixed_and_row_plans_at_wide_widths(cs, orc, torch_cuda):
+    """Products wider than one lane group of the row kernel (256 columns): its rows are walked slab by slab, on their
+    own and as the row blocks of the fused launches.  Integer operands, so every path must equal the oracle bit for bit;
+    widths that are and are not multiples of the slab, and of four."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    M, K = 320, 1024
+    dense_rows = set(range(32, 96)) | set(range(208, 240))
+    rp, cl, vl = random_csr(rng, M, K, row_nnz=lambda r: 48 if r in dense_rows else 3, values="ints")
+    for r in dense_rows:
+        s, e = int(rp[r]), int(rp[r + 1])
+        cl[s:e] = np.sort(rng.choice(np.arange((r // 16) * 8, (r // 16) * 8 + 64), e - s, replace=False)).astype(cl.dtype)
+    h = cs.HRPB(M, K, rp, cl, vl)
+    for N in (260, 512, 516, 770, 1024):
+        B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+        ref = orc.spmm_csr(rp, cl, vl, B)
+        for kw in (dict(), dict(mfma_shape=1), dict(mfma_shape=2), dict(path=cs.PATH_ROWS), dict(mfma_shape=1, brick_groups=2)):
+            out, plan = _run(cs, torch, h, B, **kw)
+            info = plan.info
+            assert (out == ref).all(), (N, kw, info)
+            if "path" not in kw:
+                assert info["numChunks"] > 0 and info["numRowPanelsSparse"] > 0, (N, kw, info)
+                if N % 4 == 0 and "brick_groups" not in kw:
+                    assert info["fusedLaunch"] == 1, (N, kw, info)
+        # the same through a row list that leaves rows out (every second panel forced to the MFMA side by its long rows)
+        plan = cs.SPMM_TC(h, N, max_row_nnz=8)
+        dB = torch.from_numpy(B).cuda()
+        dC = torch.full((M, N), float("nan"), device="cuda")
+        plan.run(dB, dC)
+        torch.cuda.synchronize()
+        assert (dC.cpu().numpy() == ref).all(), (N, plan.info)
+
+
 def test_few_huge_panels_are_still_cut(cs, orc, torch_cuda):
     """A handful of dense rows among many short ones: only their panels go to the MFMA kernel, all of
     them long.  Their mean length must not become the chunk length, or one wavefront walks a panel alone."""
